@@ -152,11 +152,22 @@ class MlstmSpec(BaseModel):
     gate_cap: float
 
 
+class SharedExpertSpec(BaseModel):
+    """A silu-GLU expert that every token passes; its output is scaled by
+    sigmoid of one more projection of the input (a scalar per token)."""
+
+    ff: int
+
+
 class RoutedExpertsSpec(BaseModel):
-    """Mixture of silu-GLU experts behind a softmax router. The last
+    """Mixture of silu-GLU experts behind a router. ``score`` turns the router
+    logits into scores: softmax over all outputs, or sigmoid of each. The last
     ``identity`` router outputs are experts that return their input. The
-    choice is made on score + correction among the experts of the best
-    ``group_keep`` of ``group_count`` groups of neighbours."""
+    choice is made on score (+ correction, if the checkpoint has one) among
+    the experts of the best ``group_keep`` of ``group_count`` groups of
+    neighbours. The chosen scores weigh the experts, renormalised to sum 1 or
+    as they are; the weight multiplies the expert's output or its input
+    (``weight_on``). ``shared``: one more expert that runs for every token."""
 
     kind: Literal["moe"] = "moe"
     experts: int
@@ -165,6 +176,11 @@ class RoutedExpertsSpec(BaseModel):
     group_count: int = 1
     group_keep: int = 1
     ff: int
+    score: Literal["softmax", "sigmoid"] = "softmax"
+    renormalize: bool = True
+    correction: bool = True
+    weight_on: Literal["output", "input"] = "output"
+    shared: Optional[SharedExpertSpec] = None
 
 
 class BigramSpec(BaseModel):
@@ -295,6 +311,136 @@ def _medilix_preset(vocab, width, depth, heads, kv_heads, dim, mask, keep, r_hea
     return MedilixArchConfig(vocab_size=vocab, hidden_size=width, norm_groups=groups, embed_scale=1.0,
                              bigram=BigramSpec(buckets=max(7, vocab // 2 - 1), mul_prev=131, mul_cur=5),
                              layers=layers, loop=LoopSpec(**loop) if loop else None)
+
+
+class LatentAttnSpec(BaseModel):
+    """Softmax attention whose keys and values are up-projections of one
+    shared latent row per token. Per head the query has ``dim`` unrotated and
+    ``rot_dim`` rotated entries; the token's down-projection gives the latent
+    (``kv_rank`` entries, RMS-normed) and one rotated key part shared by all
+    heads. Only those two are cached. Causal sliding window of ``mask_size``
+    positions (0 = plain causal); per-head sigmoid output gate."""
+
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
+    mask_size: int = 0
+    rot: RotarySpec = Field(default_factory=RotarySpec)
+    head_gate: bool = True
+
+
+class ActFFSpec(BaseModel):
+    """Two-matrix feed-forward W_down act(W_up h); act = tanh-form gelu."""
+
+    kind: Literal["dense"] = "dense"
+    ff: int
+    act: Literal["gelu_tanh"] = "gelu_tanh"
+
+
+class MitunexLayerSpec(BaseModel):
+    type: Literal["latent_attention"] = "latent_attention"
+    attention: LatentAttnSpec
+    mlp: Optional[Union[ActFFSpec, RoutedExpertsSpec]] = None
+    # index of the layer whose weights this one uses (its own index = own weights)
+    weights_of: int
+
+
+class MitunexArchConfig(BaseModel):
+    """A decoder of post-normed layers x <- x + norm(mixer(x)),
+    x <- x + norm(ff(x)) over an fp32 residual. The embedding adds a learned
+    position row and is RMS-normed. Every mixer is latent attention with a
+    sliding window; feed-forwards are a gelu layer, routed experts with
+    sigmoid scores and a shared expert, or absent. A layer may use another
+    layer's weights with a cache of its own. The logits are scaled and
+    soft-capped. Every size comes from the checkpoint's config.json."""
+
+    arch: Literal["mitunex"] = "mitunex"
+    vocab_size: int
+    hidden_size: int
+    rms_norm_eps: float = 1e-6
+    layers: List[MitunexLayerSpec]
+    max_position_embeddings: int = 2048
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0          # 0 = none
+    tie_word_embeddings: bool = False
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_checkpoint_config(cls, d: dict, shapes: Optional[dict] = None) -> "MitunexArchConfig":
+        """Parse the family's config.json (keys: vocab, width, norm.eps,
+        max_positions, logit_scale, logit_softcap, layers[].type / .mixer /
+        .mlp / .weights_of)."""
+        layers = []
+        for li, spec in enumerate(d["layers"]):
+            if spec["type"] != "latent_attention":
+                raise ValueError(f"unknown layer type {spec['type']!r}")
+            m = spec["mixer"]
+            rot = m.get("rot") or {}
+            mask = m.get("mask") or {}
+            att = LatentAttnSpec(heads=m["heads"], dim=m["dim"], rot_dim=m["rot_dim"], vdim=m["vdim"],
+                                 kv_rank=m["kv_rank"], scale=m["scale"], mask_size=mask.get("size") or 0,
+                                 rot=RotarySpec(base=rot.get("base", 10000.0), dims=rot.get("dims", m["rot_dim"])))
+            if att.rot.dims != att.rot_dim:
+                raise ValueError("the rotated part of a latent-attention head is rotated whole")
+            mlp = spec.get("mlp")
+            ff = None
+            if mlp:
+                kind = mlp.get("kind", "dense")
+                if kind == "dense":
+                    ff = ActFFSpec(ff=mlp["ff"])
+                elif kind == "moe":
+                    r = mlp["router"]
+                    sh = mlp.get("shared")
+                    ff = RoutedExpertsSpec(experts=r["experts"], top=r["top"], ff=mlp["expert"]["ff"],
+                                           score="sigmoid", renormalize=False, correction=False,
+                                           weight_on="input",
+                                           shared=SharedExpertSpec(ff=sh["ff"]) if sh else None)
+                else:
+                    raise ValueError(f"unknown feed-forward kind {kind!r}")
+            src = spec.get("weights_of", li)
+            if src is None:
+                src = li
+            if not 0 <= src < len(d["layers"]) or d["layers"][src].get("weights_of", src) not in (src, None):
+                raise ValueError(f"layer {li}: weights_of {src} does not name a layer with weights of its own")
+            layers.append(MitunexLayerSpec(attention=att, mlp=ff, weights_of=src))
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"], rms_norm_eps=d["norm"]["eps"], layers=layers,
+                   max_position_embeddings=d.get("max_positions", 2048), logit_scale=d.get("logit_scale") or 1.0,
+                   logit_softcap=d.get("logit_softcap") or 0.0)
+
+
+def _mitunex_preset(vocab, width, depth, heads, dim, rot_dim, vdim, kv_rank, mask, ff, experts, top, expert_ff,
+                    shared_ff, pattern="dm", share_from=None, max_pos=8192) -> MitunexArchConfig:
+    """Random-init presets of the family: ``pattern`` repeats over the depth
+    ('d' gelu feed-forward, 'm' routed experts + shared expert, 'n' none);
+    layers from ``share_from`` on use the weights of layer share_from - 1."""
+    import math as _math
+
+    layers = []
+    for i in range(depth):
+        c = pattern[i % len(pattern)]
+        att = LatentAttnSpec(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank,
+                             scale=1.0 / _math.sqrt(dim + rot_dim), mask_size=mask,
+                             rot=RotarySpec(base=1e6, dims=rot_dim))
+        mlp = None
+        if c == "d":
+            mlp = ActFFSpec(ff=ff)
+        elif c == "m":
+            mlp = RoutedExpertsSpec(experts=experts, top=top, ff=expert_ff, score="sigmoid", renormalize=False,
+                                    correction=False, weight_on="input",
+                                    shared=SharedExpertSpec(ff=shared_ff) if shared_ff else None)
+        src = i
+        if share_from is not None and i >= share_from:
+            src = share_from - 1
+            att, mlp = layers[src].attention, layers[src].mlp
+        layers.append(MitunexLayerSpec(attention=att, mlp=mlp, weights_of=src))
+    return MitunexArchConfig(vocab_size=vocab, hidden_size=width, layers=layers, max_position_embeddings=max_pos,
+                             logit_scale=1.5, logit_softcap=30.0)
 
 
 class HybridLayerSpec(BaseModel):
@@ -492,6 +638,21 @@ MODEL_PRESETS: dict = {
     "medilix-1b-l6": _medilix_preset(
         vocab=32000, width=2048, depth=6, heads=16, kv_heads=4, dim=128, mask=1024, keep=4, r_heads=32,
         r_dim=64, m_heads=16, m_dim=64, m_vdim=128, ff=8192, experts=8, top=2, expert_ff=4096, identity=0),
+    # Mitunex family (post-normed layers; latent attention with a sliding
+    # window; gelu and routed feed-forwards; layers that share weights)
+    "tiny-mitunex": _mitunex_preset(
+        vocab=512, width=64, depth=4, heads=4, dim=16, rot_dim=8, vdim=24, kv_rank=32, mask=24, ff=96,
+        experts=6, top=2, expert_ff=48, shared_ff=40, share_from=3, max_pos=512),
+    "mid-mitunex": _mitunex_preset(
+        vocab=2048, width=512, depth=3, heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=128, mask=256, ff=1024,
+        experts=8, top=2, expert_ff=256, shared_ff=256, max_pos=2048),
+    # layer shapes of real models at reduced depth, beside llama-/medilix-{1b,8b}-l6
+    "mitunex-8b-l6": _mitunex_preset(
+        vocab=32000, width=4096, depth=6, heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512, mask=2048,
+        ff=14336, experts=8, top=2, expert_ff=7168, shared_ff=2048),
+    "mitunex-1b-l6": _mitunex_preset(
+        vocab=32000, width=2048, depth=6, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, mask=1024,
+        ff=8192, experts=8, top=2, expert_ff=4096, shared_ff=1024),
 }
 
 
@@ -594,10 +755,11 @@ class EngineConfig(BaseModel):
         with open(cfg_path) as f:
             hf = json.load(f)
         family = str(hf.get("architecture", "")).lower()
-        if family in ("zutalix", "medilix"):
+        if family in ("zutalix", "medilix", "mitunex"):
             from .weights import safetensors_shapes
 
-            reader = HybridArchConfig if family == "zutalix" else MedilixArchConfig
+            reader = {"zutalix": HybridArchConfig, "medilix": MedilixArchConfig,
+                      "mitunex": MitunexArchConfig}[family]
             return reader.from_checkpoint_config(hf, safetensors_shapes(os.path.dirname(cfg_path)))
         arch = "mixtral" if "mixtral" in hf.get("model_type", "").lower() or hf.get("num_local_experts") else "llama"
         return ModelArchConfig(

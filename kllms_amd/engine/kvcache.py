@@ -208,7 +208,8 @@ class PagedKVCache:
 @dataclass
 class LayerCacheSpec:
     """What one layer keeps between steps. kv = (kv_heads, key_dim, value_dim)
-    of a paged attention cache; rec = (heads, key_dim, value_dim) of an fp32
+    of a paged attention cache (value_dim 0: the layer's values are read from
+    its key rows, as latent attention does, and the value tensor is empty); rec = (heads, key_dim, value_dim) of an fp32
     recurrent state matrix per head; conv = (channels, history) of carried
     convolution inputs; shift = width of the previous token's layer input
     (token-shift mixers); tok = the previous token id (hashed n-gram

@@ -2,7 +2,8 @@
 parameters: block-local softmax attention over the paged cache, decayed
 linear attention, the gated delta rule with per-channel decay and short
 convolutions, the clamped GLU; windowed attention with kept first tokens and
-a sink, the wkv and mlstm recurrences, and routed experts. Each runs on "segment" batches
+a sink, the wkv and mlstm recurrences, routed experts; latent attention and
+the two-matrix gelu feed-forward. Each runs on "segment" batches
 (ForwardBatch.seg_start / state_slots / token_seg): any mix of prompt
 portions and single decoded tokens, attention keys found through the block
 table and recurrent state carried in per-sequence slots.
@@ -23,8 +24,9 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import ops
-from ..engine.config import (BlockAttnSpec, ChannelDeltaSpec, DecayLinearAttnSpec, GluSpec, MaskedAttnSpec,
-                             MlstmSpec, ParallelMixerSpec, RotarySpec, RoutedExpertsSpec, WkvSpec)
+from ..engine.config import (ActFFSpec, BlockAttnSpec, ChannelDeltaSpec, DecayLinearAttnSpec, GluSpec,
+                             LatentAttnSpec, MaskedAttnSpec, MlstmSpec, ParallelMixerSpec, RotarySpec,
+                             RoutedExpertsSpec, WkvSpec)
 from ..engine.kvcache import LayerCacheSpec, LayerState
 
 
@@ -381,6 +383,84 @@ class WindowSinkAttention(nn.Module):
         return m
 
 
+class LatentAttention(nn.Module):
+    """Softmax attention over one shared latent row per token. The input's
+    down-projection gives the latent c (RMS-normed, kv_rank wide) and one
+    rotated key part shared by the heads; only [c | rotated part] is cached
+    (one paged row per token). Per head the key is [W_uk c | rotated part] and
+    the value W_uv c, so with q = [q_n | q_r]
+        score_j = (q_n . W_uk c_j + q_r . kr_j) scale = ((W_uk^T q_n) . c_j + q_r . kr_j) scale
+        out     = W_uv sum_j p_j c_j
+    and the attention proper runs in the latent space for all heads against
+    the same cached rows: W_uk is applied to the queries before it (one
+    batched product over the heads) and W_uv to its result. Sliding causal
+    window, per-head sigmoid output gate; q, the down-projection and the gate
+    share one input GEMM."""
+
+    def __init__(self, spec: LatentAttnSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        assert spec.rot.dims == spec.rot_dim and spec.rot_dim % 2 == 0
+        self.spec = spec
+        self.eps = eps
+        H, D, R, V, C = spec.heads, spec.dim, spec.rot_dim, spec.vdim, spec.kv_rank
+        parts = [("q", H * (D + R)), ("dkv", C + R)]
+        if spec.head_gate:
+            parts.append(("g", H))
+        self.inp = FusedInput(hidden, parts, dtype)
+        self.dkv_norm = _param(C, dtype=torch.float32)
+        self.uk = _param(H, D, C, dtype=dtype)
+        self.uv = _param(H, V, C, dtype=dtype)
+        self.o_proj = _param(hidden, H * V, dtype=dtype)
+        self.register_buffer("inv_freq", rotary_inv_freq(spec.rot), persistent=False)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        return LayerCacheSpec(kv=(1, sp.kv_rank + sp.rot_dim, 0))
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        T = h.shape[0]
+        H, D, R, V = sp.heads, sp.dim, sp.rot_dim, sp.vdim
+        y = self.inp(h)
+        s = self.inp.split
+        q = s(y, "q").unflatten(1, (H, D + R))
+        ops.latent_kv_store(q, s(y, "dkv"), self.dkv_norm, self.eps, batch.positions, self.inv_freq, st.k,
+                            batch.slot_mapping, D)
+        q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk)                   # [H, T, C]
+        lat = ops.attn_latent_paged(q_abs.transpose(0, 1), q, st.k, batch.block_tables, batch.token_seg,
+                                    batch.positions, sp.scale, sp.mask_size,
+                                    s(y, "g") if sp.head_gate else None, D,
+                                    tile_rows=1 if batch.host_segs is not None
+                                    and all(n == 1 for _, n in batch.host_segs) else 0)       # [T, H, C]
+        att = torch.empty((T, H * V), dtype=y.dtype, device=y.device)
+        torch.bmm(lat.transpose(0, 1), self.uv.transpose(1, 2), out=att.view(T, H, V).transpose(0, 1))
+        return F.linear(att, self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
+        m[pre + "dkv.norm"] = self.dkv_norm
+        m[pre + "uk"] = self.uk.view(-1, self.spec.kv_rank)
+        m[pre + "uv"] = self.uv.view(-1, self.spec.kv_rank)
+        m[pre + "o"] = self.o_proj
+        return m
+
+
+class ActFF(nn.Module):
+    """y = W_down act(W_up h) with the tanh-form gelu."""
+
+    def __init__(self, spec: ActFFSpec, hidden: int, dtype):
+        super().__init__()
+        self.spec = spec
+        self.up = _param(spec.ff, hidden, dtype=dtype)
+        self.down = _param(hidden, spec.ff, dtype=dtype)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return F.linear(ops.gelu_tanh(F.linear(h, self.up)), self.down)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        return {pre + "up": self.up, pre + "down": self.down}
+
+
 class WkvMixer(nn.Module):
     """Time mixing with token shift. With h' the previous token's input, each
     of r, k, v, g, w reads h + (h' - h) mu_s; r, k, v are projections of their
@@ -490,10 +570,13 @@ class MlstmMixer(nn.Module):
 
 class RoutedExperts(nn.Module):
     """Mixture of silu-GLU experts. The router runs in fp32: scores are the
-    softmax over all outputs; the choice is made on score + correction within
-    the best groups of neighbouring experts; the chosen scores, renormalised,
-    weigh the outputs. The last ``identity`` router outputs stand for experts
-    that return their input and have no weights.
+    softmax over all outputs or the sigmoid of each; the choice is made on
+    score (+ correction) within the best groups of neighbouring experts; the
+    chosen scores, renormalised or as they are, weigh the experts — their
+    outputs, or (``weight_on = "input"``) their inputs: expert(w h). The last
+    ``identity`` router outputs stand for experts that return their input and
+    have no weights. An optional shared expert runs for every row and is
+    added times sigmoid of one more projection of the row.
 
     Few rows (decode): every expert runs on every row as two batched GEMMs
     (the weights stream from memory once either way, and shapes do not depend
@@ -517,45 +600,74 @@ class RoutedExperts(nn.Module):
         n = spec.experts + spec.identity
         assert n % spec.group_count == 0 and 1 <= spec.group_keep <= spec.group_count
         assert spec.top <= n // spec.group_count * spec.group_keep
+        assert not (spec.weight_on == "input" and spec.identity), "identity experts take their weight on the output"
         self.router = _param(n, hidden, dtype=torch.float32)
-        self.correction = _param(n, dtype=torch.float32)
+        self.correction = _param(n, dtype=torch.float32) if spec.correction else None
         self.w_gate_up = _param(spec.experts, 2 * spec.ff, hidden, dtype=dtype)
         self.w_down = _param(spec.experts, hidden, spec.ff, dtype=dtype)
+        self.shared_inp = self.shared_down = None
+        if spec.shared is not None:
+            sff = spec.shared.ff
+            self.shared_inp = FusedInput(hidden, [("gate", sff), ("up", sff), ("sg", 1)], dtype)
+            self.shared_down = _param(hidden, sff, dtype=dtype)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         sp = self.spec
         T, W = h.shape
         E, top = sp.experts, sp.top
+        on_input = sp.weight_on == "input"
         dense = T <= self.DENSE_MAX_ROWS and E * T <= self.DENSE_MAX_PAIRS
         idx, w, rowidx = ops.moe_route_rows(h, self.router, self.correction, top, sp.group_count, sp.group_keep,
-                                            E, dense)
+                                            E, dense, sp.score, sp.renormalize)
         if dense:
-            gu = torch.bmm(h.unsqueeze(0).expand(E, T, W), self.w_gate_up.transpose(1, 2)).view(E * T, 2 * sp.ff)
+            if on_input:
+                # expert e reads w[t, e] h[t] where it was chosen (zero rows elsewhere; they are never read back)
+                wsel = torch.zeros((T, E), dtype=torch.float32, device=h.device).scatter_(1, idx.long(), w)
+                src = torch.arange(T, dtype=torch.int32, device=h.device).repeat(E)
+                xin = ops.scale_rows(h, src, wsel.t().reshape(-1)).view(E, T, W)
+            else:
+                xin = h.unsqueeze(0).expand(E, T, W)
+            gu = torch.bmm(xin, self.w_gate_up.transpose(1, 2)).view(E * T, 2 * sp.ff)
             act = ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]).view(E, T, sp.ff)
             rows = torch.bmm(act, self.w_down.transpose(1, 2)).view(E * T, W)
-            return ops.moe_combine(rows, h, rowidx, w, h.dtype)
-        flat = idx.reshape(-1).long().clamp(max=E)                # identity experts sort last
-        order = torch.argsort(flat, stable=True)
-        counts = torch.bincount(flat, minlength=E + 1)[:E].tolist()   # one host sync per call
-        n_real = sum(counts)
-        xs = h[(order[:n_real] // top)]
-        rows = torch.empty((max(n_real, 1), W), dtype=h.dtype, device=h.device)
-        s0 = 0
-        for e, c in enumerate(counts):
-            if c:
-                gu = F.linear(xs[s0:s0 + c], self.w_gate_up[e])
-                rows[s0:s0 + c] = F.linear(ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]), self.w_down[e])
-                s0 += c
-        pos = torch.empty(T * top, dtype=torch.int32, device=h.device)
-        pos[order] = torch.arange(T * top, dtype=torch.int32, device=h.device)
-        rowidx = torch.where(idx < E, pos.view(T, top), torch.full_like(idx, -1))
-        return ops.moe_combine(rows, h, rowidx, w, h.dtype)
+        else:
+            flat = idx.reshape(-1).long().clamp(max=E)                # identity experts sort last
+            order = torch.argsort(flat, stable=True)
+            counts = torch.bincount(flat, minlength=E + 1)[:E].tolist()   # one host sync per call
+            n_real = sum(counts)
+            if on_input:
+                xs = ops.scale_rows(h, (order[:n_real] // top).int(), w.reshape(-1)[order[:n_real]])
+            else:
+                xs = h[(order[:n_real] // top)]
+            rows = torch.empty((max(n_real, 1), W), dtype=h.dtype, device=h.device)
+            s0 = 0
+            for e, c in enumerate(counts):
+                if c:
+                    gu = F.linear(xs[s0:s0 + c], self.w_gate_up[e])
+                    rows[s0:s0 + c] = F.linear(ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]), self.w_down[e])
+                    s0 += c
+            pos = torch.empty(T * top, dtype=torch.int32, device=h.device)
+            pos[order] = torch.arange(T * top, dtype=torch.int32, device=h.device)
+            rowidx = torch.where(idx < E, pos.view(T, top), torch.full_like(idx, -1))
+        extra = gate = None
+        if self.shared_inp is not None:
+            ys = self.shared_inp(h)
+            ss = self.shared_inp.split
+            extra = F.linear(ops.silu_glu(ss(ys, "gate"), ss(ys, "up")), self.shared_down)
+            gate = ss(ys, "sg")[:, 0]
+        return ops.moe_combine(rows, h, rowidx, None if on_input else w, h.dtype, extra, gate)
 
     def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
         ff = self.spec.ff
-        m = {pre + "router": self.router, pre + "correction": self.correction}
+        m = {pre + "router": self.router}
+        if self.correction is not None:
+            m[pre + "correction"] = self.correction
         for e in range(self.spec.experts):
             m[f"{pre}e{e}.gate"] = self.w_gate_up[e, :ff]
             m[f"{pre}e{e}.up"] = self.w_gate_up[e, ff:]
             m[f"{pre}e{e}.down"] = self.w_down[e]
+        if self.shared_inp is not None:
+            for n in ("gate", "up", "sg"):
+                m[f"{pre}shared.{n}"] = self.shared_inp.slot(n)
+            m[pre + "shared.down"] = self.shared_down
         return m

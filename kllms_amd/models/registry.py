@@ -22,7 +22,11 @@ def model_class(arch: str):
         from .medilix import MedilixForCausalLM
 
         return MedilixForCausalLM
+    if arch == "mitunex":
+        from .mitunex import MitunexForCausalLM
+
+        return MitunexForCausalLM
     raise ValueError(f"no model registered for architecture {arch!r}")
 
 
-ARCHITECTURES = ("llama", "mixtral", "zutalix", "medilix")
+ARCHITECTURES = ("llama", "mixtral", "zutalix", "medilix", "mitunex")

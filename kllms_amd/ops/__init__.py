@@ -244,12 +244,15 @@ def _none(ref: torch.Tensor, dtype=None) -> torch.Tensor:
     return torch.empty(0, dtype=dtype or ref.dtype, device=ref.device)
 
 
-def embed_rmsnorm(ids, table, weight, eps):
+def embed_rmsnorm(ids, table, weight, eps, pos_table=None, positions=None):
+    """fp32 rms(table[ids] (+ pos_table[positions])) * weight."""
     if _gpu(table):
         out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
-        _seq().embed_rmsnorm(out, ids, table, weight, eps)
+        has = pos_table is not None
+        _seq().embed_rmsnorm(out, ids, table, weight, eps, pos_table if has else _none(table),
+                             positions if has else _none(table, torch.long))
         return out
-    return torch_ref.embed_rmsnorm(ids, table, weight, eps)
+    return torch_ref.embed_rmsnorm(ids, table, weight, eps, pos_table, positions)
 
 
 def rmsnorm_cast(x, weight, eps, out_dtype):
@@ -260,18 +263,20 @@ def rmsnorm_cast(x, weight, eps, out_dtype):
     return torch_ref.rmsnorm_cast(x, weight, eps, out_dtype)
 
 
-def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, out_dtype=None):
+def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, out_dtype=None, cast=False):
     """x (fp32 residual, in place) += rms(y) * w_post with y = a, or
-    y = (rms(a) wa + rms(b) wb) / 2; returns rms(x) * w_next in out_dtype
-    (None when w_next is None)."""
+    y = (rms(a) wa + rms(b) wb) / 2; returns rms(x) * w_next in a's dtype.
+    With w_next None: the new x in a's dtype if ``cast`` (the input of a
+    sublayer that reads the stream itself), else None."""
     if _gpu(x):
-        out = torch.empty(a.shape, dtype=a.dtype, device=a.device) if w_next is not None else _none(a)
+        want = w_next is not None or cast
+        out = torch.empty(a.shape, dtype=a.dtype, device=a.device) if want else _none(a)
         f = _none(x, torch.float32)
         _seq().sandwich_residual(
             x, a, b if b is not None else _none(a), wa if b is not None else f, wb if b is not None else f,
             w_post, w_next if w_next is not None else f, out, eps)
-        return out if w_next is not None else None
-    return torch_ref.sandwich_residual(x, a, w_post, eps, b, wa, wb, w_next, out_dtype or a.dtype)
+        return out if want else None
+    return torch_ref.sandwich_residual(x, a, w_post, eps, b, wa, wb, w_next, out_dtype or a.dtype, cast)
 
 
 def rope_pairs_store(q, k, v, positions, inv_freq, k_cache, v_cache, slot_mapping, kv_fresh=None) -> None:
@@ -504,18 +509,20 @@ def head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype):
     return torch_ref.head_rmsnorm_gate(o, weight, gate, eps, gate_act, out_dtype)
 
 
-def moe_route(z, correction, top, group_count, group_keep):
+def moe_route(z, correction, top, group_count, group_keep, score="softmax", renormalize=True):
     """Routing from fp32 logits z [T, N]: (idx [T, top] int32, w [T, top] fp32)."""
     if _gpu(z):
         idx = torch.empty((z.shape[0], top), dtype=torch.int32, device=z.device)
         w = torch.empty((z.shape[0], top), dtype=torch.float32, device=z.device)
-        _seq().moe_route(idx, w, _none(z, torch.int32), z, _none(z), correction, int(top), int(group_count),
-                         int(group_keep), 0)
+        _seq().moe_route(idx, w, _none(z, torch.int32), z, _none(z),
+                         correction if correction is not None else _none(z), int(top), int(group_count),
+                         int(group_keep), 0, 0 if score == "softmax" else 1, bool(renormalize))
         return idx, w
-    return torch_ref.moe_route(z, correction, top, group_count, group_keep)
+    return torch_ref.moe_route(z, correction, top, group_count, group_keep, score, renormalize)
 
 
-def moe_route_rows(h, router, correction, top, group_count, group_keep, experts, all_experts_form):
+def moe_route_rows(h, router, correction, top, group_count, group_keep, experts, all_experts_form,
+                   score="softmax", renormalize=True):
     """Router GEMV in fp32 + routing in one kernel. Returns (idx, w, rowidx);
     rowidx [T, top] (only when all_experts_form) addresses rows of the
     all-experts output [experts * T, W]: choice * T + row, -1 = identity."""
@@ -524,11 +531,13 @@ def moe_route_rows(h, router, correction, top, group_count, group_keep, experts,
         idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
         w = torch.empty((T, top), dtype=torch.float32, device=h.device)
         rowidx = torch.empty((T, top), dtype=torch.int32, device=h.device) if all_experts_form else None
-        _seq().moe_route(idx, w, rowidx if rowidx is not None else _none(h, torch.int32), h, router, correction,
-                         int(top), int(group_count), int(group_keep), int(experts))
+        _seq().moe_route(idx, w, rowidx if rowidx is not None else _none(h, torch.int32), h, router,
+                         correction if correction is not None else _none(router),
+                         int(top), int(group_count), int(group_keep), int(experts),
+                         0 if score == "softmax" else 1, bool(renormalize))
         return idx, w, rowidx
     z = torch.nn.functional.linear(h.float(), router)
-    idx, w = torch_ref.moe_route(z, correction, top, group_count, group_keep)
+    idx, w = torch_ref.moe_route(z, correction, top, group_count, group_keep, score, renormalize)
     rowidx = None
     if all_experts_form:
         t_idx = torch.arange(T, dtype=torch.int32, device=h.device).unsqueeze(1)
@@ -536,12 +545,73 @@ def moe_route_rows(h, router, correction, top, group_count, group_keep, experts,
     return idx, w, rowidx
 
 
-def moe_combine(rows, h, rowidx, w, out_dtype):
+def moe_combine(rows, h, rowidx, w, out_dtype, extra=None, extra_gate=None):
+    """Fixed-order sum of each row's chosen expert rows, weighted by w (None =
+    unweighted), plus sigmoid(extra_gate[t]) * extra[t] when given
+    (extra_gate: a [T] view, any stride)."""
     if _gpu(h):
         out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
-        _seq().moe_combine(out, rows, h, rowidx, w)
+        _seq().moe_combine(out, rows, h, rowidx, w if w is not None else _none(h, torch.float32),
+                           extra if extra is not None else _none(h),
+                           extra_gate if extra is not None else _none(h))
         return out
-    return torch_ref.moe_combine(rows, h, rowidx, w, out_dtype)
+    return torch_ref.moe_combine(rows, h, rowidx, w, out_dtype, extra, extra_gate)
+
+
+def scale_rows(h, src_row, scale):
+    """out[i] = h[src_row[i]] * scale[i]: expert inputs that carry their
+    routing weight. src_row int32 [n], scale fp32 [n]."""
+    if _gpu(h):
+        out = torch.empty((src_row.numel(), h.shape[1]), dtype=h.dtype, device=h.device)
+        _seq().scale_rows(out, h, src_row, scale)
+        return out
+    return torch_ref.scale_rows(h, src_row, scale)
+
+
+def gelu_tanh(x):
+    """Tanh-form gelu of a [T, C] row view, in x's dtype."""
+    if _gpu(x):
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _seq().gelu_tanh(out, x)
+        return out
+    return torch_ref.gelu_tanh(x)
+
+
+def scale_softcap_(z, scale: float, cap: float) -> None:
+    """fp32 logits in place: z * scale, then cap * tanh(. / cap) if cap > 0."""
+    if _gpu(z):
+        _seq().scale_softcap(z, float(scale), float(cap))
+        return
+    torch_ref.scale_softcap_(z, scale, cap)
+
+
+def latent_kv_store(q, dkv, w_norm, eps, positions, inv_freq, cache, slot_mapping, nope_dim) -> None:
+    """Rotates the rotated part of every query head in place; norms the
+    latent, rotates the shared key part and stores [latent | key part] into
+    the paged latent cache."""
+    if _gpu(q):
+        _seq().latent_kv_store(q, dkv, w_norm, eps, positions, inv_freq, cache, slot_mapping, int(nope_dim))
+        return
+    torch_ref.latent_kv_store(q, dkv, w_norm, eps, positions, inv_freq, cache, slot_mapping, nope_dim)
+
+
+def attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale, mask_size, gate, nope_dim,
+                      tile_rows: int = 0, use_mfma: bool = True):
+    """Sliding-window softmax attention over the paged latent cache in the
+    absorbed form (one shared key/value row per token for all heads):
+    returns the heads' weighted latent sums [T, H, C], gated per head.
+    GPU: bf16 rows go through the matrix-unit kernel when the sizes fit it
+    (``tile_rows`` = query rows per workgroup, 0 = as many as fit 32 (row,
+    head) columns; 1 suits steps of single decoded tokens), fp32 rows and
+    other sizes through the plain kernel."""
+    if _gpu(q):
+        out = torch.empty((q.shape[0], q.shape[1], q_abs.shape[2]), dtype=q.dtype, device=q.device)
+        _seq().attn_latent_paged(out, q_abs, q, cache, block_tables, token_seg, positions,
+                                 gate if gate is not None else _none(q), float(scale), int(mask_size),
+                                 int(nope_dim), int(tile_rows), bool(use_mfma))
+        return out
+    return torch_ref.attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale, mask_size,
+                                       gate, nope_dim)
 
 
 def attn_window_sink(q, st, batch, spec, gate):

@@ -8,7 +8,16 @@
 #include <hip/hip_bf16.h>
 
 extern "C" {
-void seq_launch_embed_rmsnorm(float*, const int64_t*, const void*, const float*, int, int, float, int, hipStream_t);
+void seq_launch_embed_rmsnorm(float*, const int64_t*, const void*, const float*, const void*, const int64_t*, int,
+                              int, float, int, hipStream_t);
+void seq_launch_gelu_tanh(void*, const void*, int64_t, int, int, int, hipStream_t);
+void seq_launch_scale_softcap(float*, int64_t, float, float, hipStream_t);
+void seq_launch_scale_rows(void*, const void*, const int*, const float*, int, int, int, hipStream_t);
+void seq_launch_latent_kv_store(void*, const void*, const float*, float, const int64_t*, const float*, void*,
+                                const int64_t*, int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_attn_latent_paged(void*, const void*, const void*, const void*, const int*, const int*,
+                                  const int64_t*, const void*, float, int, int, int, int, int, int, int, int,
+                                  int64_t, int64_t, int, int, int, int, int, hipStream_t);
 void seq_launch_rmsnorm_cast(void*, const float*, const float*, int, int, float, int, hipStream_t);
 void seq_launch_sandwich_residual(float*, const void*, const void*, const float*, const float*, const float*,
                                   const float*, void*, int, int, float, int, hipStream_t);
@@ -34,9 +43,9 @@ void seq_launch_head_rmsnorm_gate(void*, const float*, const float*, const void*
 void seq_launch_token_shift_mix(void*, float*, const void*, const float*, void*, const int*, const int*,
                                 const int*, const int*, int, int, int, int, int, int, hipStream_t);
 void seq_launch_moe_route(int*, float*, int*, const float*, const void*, const float*, const float*, int, int, int,
-                          int, int, int, int, int, hipStream_t);
-void seq_launch_moe_combine(void*, const void*, const void*, const int*, const float*, int, int, int, int,
-                            hipStream_t);
+                          int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_moe_combine(void*, const void*, const void*, const int*, const float*, const void*, const void*,
+                            int, int, int, int, int, hipStream_t);
 void seq_launch_wkv_recurrence(float*, const void*, const void*, const void*, const float*, const float*,
                                const float*, float*, float*, float*, float*, float*, float*, const int*,
                                const int*, const int*, int, int, int, int, int, int, int, int, int, hipStream_t);
@@ -82,14 +91,96 @@ static int f32flag(const torch::Tensor& t) { return t.scalar_type() == at::kFloa
 #define CHECK_ROWS3(t) \
   TORCH_CHECK((t).dim() == 3 && (t).stride(2) == 1 && (t).stride(1) == (t).size(2), #t " must be a [T, H, D] row view")
 
-void embed_rmsnorm(torch::Tensor out, torch::Tensor ids, torch::Tensor table, torch::Tensor w, double eps) {
+// pos_table / positions: empty tensors for an embedding without position rows
+void embed_rmsnorm(torch::Tensor out, torch::Tensor ids, torch::Tensor table, torch::Tensor w, double eps,
+                   torch::Tensor pos_table, torch::Tensor positions) {
   CHECK_F32C(out); CHECK_I64C(ids); CHECK_ACT(table); CHECK_F32C(w);
   TORCH_CHECK(table.is_contiguous() && table.dim() == 2);
   const int T = ids.numel(), W = table.size(1);
   TORCH_CHECK(out.numel() == (int64_t)T * W && w.numel() == W);
+  const bool pos = pos_table.numel() > 0;
+  if (pos) {
+    CHECK_ACT(pos_table); CHECK_SAME(pos_table, table); CHECK_I64C(positions);
+    TORCH_CHECK(pos_table.is_contiguous() && pos_table.dim() == 2 && pos_table.size(1) == W && positions.numel() == T);
+  }
   if (T == 0) return;
   seq_launch_embed_rmsnorm(out.data_ptr<float>(), ids.data_ptr<int64_t>(), table.data_ptr(),
-                           w.data_ptr<float>(), T, W, (float)eps, f32flag(table), cur_stream());
+                           w.data_ptr<float>(), pos ? pos_table.data_ptr() : nullptr,
+                           pos ? positions.data_ptr<int64_t>() : nullptr, T, W, (float)eps, f32flag(table),
+                           cur_stream());
+}
+
+void gelu_tanh(torch::Tensor out, torch::Tensor x) {
+  CHECK_ACT(out); CHECK_ACT(x); CHECK_SAME(x, out); CHECK_ROWS2(x);
+  TORCH_CHECK(out.is_contiguous() && out.numel() == x.numel());
+  if (x.numel() == 0) return;
+  seq_launch_gelu_tanh(out.data_ptr(), x.data_ptr(), x.size(0), (int)x.size(1), (int)x.stride(0), f32flag(out),
+                       cur_stream());
+}
+
+void scale_softcap(torch::Tensor z, double scale, double cap) {
+  CHECK_F32C(z);
+  if (z.numel() == 0) return;
+  seq_launch_scale_softcap(z.data_ptr<float>(), z.numel(), (float)scale, (float)cap, cur_stream());
+}
+
+void scale_rows(torch::Tensor out, torch::Tensor h, torch::Tensor src_row, torch::Tensor scale) {
+  CHECK_ACT(out); CHECK_ACT(h); CHECK_SAME(h, out); CHECK_I32C(src_row); CHECK_F32C(scale);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && out.dim() == 2 && out.is_contiguous());
+  const int n = src_row.numel(), W = h.size(1);
+  TORCH_CHECK(out.size(0) == n && out.size(1) == W && scale.numel() == n);
+  if (n == 0) return;
+  seq_launch_scale_rows(out.data_ptr(), h.data_ptr(), src_row.data_ptr<int>(), scale.data_ptr<float>(), n, W,
+                        f32flag(out), cur_stream());
+}
+
+// q [T, H, D + R] row view (rotated in place), dkv [T, C + R] row view,
+// cache [NB, 1, BS, C + R] contiguous
+void latent_kv_store(torch::Tensor q, torch::Tensor dkv, torch::Tensor w, double eps, torch::Tensor positions,
+                     torch::Tensor inv_freq, torch::Tensor cache, torch::Tensor slots, int64_t nope_dim) {
+  CHECK_ACT(q); CHECK_ROWS3(q); CHECK_ACT(dkv); CHECK_SAME(dkv, q); CHECK_ROWS2(dkv); CHECK_F32C(w);
+  CHECK_I64C(positions); CHECK_F32C(inv_freq); CHECK_ACT(cache); CHECK_SAME(cache, q); CHECK_I64C(slots);
+  const int T = q.size(0), H = q.size(1), D = (int)nope_dim, R = (int)q.size(2) - D;
+  const int C = (int)dkv.size(1) - R;
+  TORCH_CHECK(D >= 0 && R >= 0 && R % 2 == 0 && C >= 1 && inv_freq.numel() == R / 2 && w.numel() == C);
+  TORCH_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == 1 && cache.size(3) == C + R);
+  TORCH_CHECK(dkv.size(0) == T && positions.numel() == T && slots.numel() == T);
+  if (T == 0) return;
+  seq_launch_latent_kv_store(q.data_ptr(), dkv.data_ptr(), w.data_ptr<float>(), (float)eps,
+                             positions.data_ptr<int64_t>(), inv_freq.data_ptr<float>(), cache.data_ptr(),
+                             slots.data_ptr<int64_t>(), T, H, D, R, C, (int)q.stride(0), (int)dkv.stride(0),
+                             f32flag(q), cur_stream());
+}
+
+// out [T, H, C] contiguous; q_abs [T, H, C] with free row and head strides;
+// q [T, H, D + R] row view; gate [T, H] row view or empty; tile_rows: rows per
+// workgroup of the matrix-unit kernel (0 = as many as fit), use_mfma false =
+// the plain kernel
+void attn_latent_paged(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q, torch::Tensor cache,
+                       torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
+                       torch::Tensor gate, double scale, int64_t mask_size, int64_t nope_dim, int64_t tile_rows,
+                       bool use_mfma) {
+  CHECK_ACT(out); CHECK_ACT(q_abs); CHECK_SAME(q_abs, out); CHECK_ACT(q); CHECK_SAME(q, out); CHECK_ROWS3(q);
+  CHECK_ACT(cache); CHECK_SAME(cache, out); CHECK_I32C(token_seg); CHECK_I64C(positions);
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
+              block_tables.stride(1) == 1);
+  const int T = q.size(0), H = q.size(1), D = (int)nope_dim, R = (int)q.size(2) - D;
+  TORCH_CHECK(q_abs.dim() == 3 && q_abs.size(0) == T && q_abs.size(1) == H && q_abs.stride(2) == 1);
+  const int C = q_abs.size(2);
+  TORCH_CHECK(D >= 0 && R >= 0 && C >= 1 && C <= 1024, "latent size out of range for the attention kernel");
+  TORCH_CHECK(cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == 1 && cache.size(3) == C + R);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 3 && out.size(0) == T && out.size(1) == H && out.size(2) == C);
+  TORCH_CHECK(token_seg.numel() == T && positions.numel() == T && mask_size >= 0);
+  TORCH_CHECK((size_t)(C + R + 128) * 4 <= 64 * 1024);
+  const bool g = gate.numel() > 0;
+  if (g) { CHECK_ACT(gate); CHECK_SAME(gate, out); CHECK_ROWS2(gate); TORCH_CHECK(gate.size(0) == T && gate.size(1) == H); }
+  if (T == 0) return;
+  seq_launch_attn_latent_paged(out.data_ptr(), q_abs.data_ptr(), q.data_ptr(), cache.data_ptr(),
+                               block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
+                               positions.data_ptr<int64_t>(), g ? gate.data_ptr() : nullptr, (float)scale,
+                               (int)mask_size, T, H, D, R, C, (int)cache.size(2), (int)block_tables.stride(0),
+                               q_abs.stride(0), q_abs.stride(1), (int)q.stride(0), g ? (int)gate.stride(0) : 0,
+                               (int)tile_rows, use_mfma ? 1 : 0, f32flag(out), cur_stream());
 }
 
 void rmsnorm_cast(torch::Tensor out, torch::Tensor x, torch::Tensor w, double eps) {
@@ -116,15 +207,18 @@ void sandwich_residual(torch::Tensor x, torch::Tensor a, torch::Tensor b, torch:
     TORCH_CHECK(b.is_cuda() && b.is_contiguous() && b.numel() == a.numel() && wa.numel() == W && wb.numel() == W);
   }
   const bool next = w_next.numel() > 0;
-  if (next) {
-    CHECK_F32C(w_next); CHECK_SAME(out, a);
-    TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.numel() == x.numel() && w_next.numel() == W);
+  const bool want = out.numel() > 0;            // without w_next: the stream itself, cast
+  TORCH_CHECK(want || !next, "w_next needs an output tensor");
+  if (next) { CHECK_F32C(w_next); TORCH_CHECK(w_next.numel() == W); }
+  if (want) {
+    CHECK_SAME(out, a);
+    TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.numel() == x.numel());
   }
   if (T == 0) return;
   seq_launch_sandwich_residual(x.data_ptr<float>(), a.data_ptr(), dual ? b.data_ptr() : nullptr,
                                dual ? wa.data_ptr<float>() : nullptr, dual ? wb.data_ptr<float>() : nullptr,
                                w_post.data_ptr<float>(), next ? w_next.data_ptr<float>() : nullptr,
-                               next ? out.data_ptr() : nullptr, T, W, (float)eps, f32flag(a), cur_stream());
+                               want ? out.data_ptr() : nullptr, T, W, (float)eps, f32flag(a), cur_stream());
 }
 
 void gated_rmsnorm(torch::Tensor out, torch::Tensor o, torch::Tensor w, torch::Tensor gate, double eps) {
@@ -451,11 +545,16 @@ void token_shift_mix(torch::Tensor act, torch::Tensor f32, torch::Tensor h, torc
 // x: fp32 logits [T, N] (router empty), or the rows h [T, W] with router [N, W] fp32 — then the logits are
 // computed in the kernel. rowidx: empty, or [T, top] for the all-experts form over `experts` real experts.
 void moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor rowidx, torch::Tensor x, torch::Tensor router,
-               torch::Tensor corr, int64_t top, int64_t gc, int64_t gk, int64_t experts) {
-  CHECK_I32C(idx); CHECK_F32C(w); CHECK_F32C(corr);
+               torch::Tensor corr, int64_t top, int64_t gc, int64_t gk, int64_t experts, int64_t score_kind,
+               bool renorm) {
+  CHECK_I32C(idx); CHECK_F32C(w);
   TORCH_CHECK(x.dim() == 2 && x.is_cuda() && x.is_contiguous());
   const bool fused = router.numel() > 0;
-  const int T = x.size(0), N = corr.numel();
+  const bool has_corr = corr.numel() > 0;          // empty: the choice is made on the plain scores
+  if (has_corr) CHECK_F32C(corr);
+  const int T = x.size(0), N = fused ? router.size(0) : x.size(1);
+  TORCH_CHECK(!has_corr || corr.numel() == N);
+  TORCH_CHECK(score_kind == 0 || score_kind == 1);
   int W = 0;
   if (fused) {
     CHECK_ACT(x); CHECK_F32C(router);
@@ -473,20 +572,32 @@ void moe_route(torch::Tensor idx, torch::Tensor w, torch::Tensor rowidx, torch::
   if (T == 0) return;
   seq_launch_moe_route(idx.data_ptr<int>(), w.data_ptr<float>(), rows ? rowidx.data_ptr<int>() : nullptr,
                        fused ? nullptr : x.data_ptr<float>(), fused ? x.data_ptr() : nullptr,
-                       fused ? router.data_ptr<float>() : nullptr, corr.data_ptr<float>(), T, N, W, (int)top,
-                       (int)gc, (int)gk, (int)experts, fused ? f32flag(x) : 1, cur_stream());
+                       fused ? router.data_ptr<float>() : nullptr, has_corr ? corr.data_ptr<float>() : nullptr, T,
+                       N, W, (int)top, (int)gc, (int)gk, (int)experts, (int)score_kind, renorm ? 1 : 0,
+                       fused ? f32flag(x) : 1, cur_stream());
 }
 
-void moe_combine(torch::Tensor out, torch::Tensor rows, torch::Tensor h, torch::Tensor rowidx, torch::Tensor w) {
+// w: empty = unweighted; extra [T, W] / extra_gate ([T] view, any stride): empty = none
+void moe_combine(torch::Tensor out, torch::Tensor rows, torch::Tensor h, torch::Tensor rowidx, torch::Tensor w,
+                 torch::Tensor extra, torch::Tensor extra_gate) {
   CHECK_ACT(out); CHECK_ACT(rows); CHECK_ACT(h); CHECK_SAME(rows, out); CHECK_SAME(h, out);
-  CHECK_I32C(rowidx); CHECK_F32C(w);
+  CHECK_I32C(rowidx);
   TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && rows.dim() == 2 && rows.is_contiguous() && out.is_contiguous());
   const int T = h.size(0), W = h.size(1), top = rowidx.size(1);
-  TORCH_CHECK(rows.size(1) == W && out.numel() == h.numel() && rowidx.dim() == 2 && rowidx.size(0) == T &&
-              w.numel() == rowidx.numel());
+  TORCH_CHECK(rows.size(1) == W && out.numel() == h.numel() && rowidx.dim() == 2 && rowidx.size(0) == T);
+  const bool weighted = w.numel() > 0;
+  if (weighted) { CHECK_F32C(w); TORCH_CHECK(w.numel() == rowidx.numel()); }
+  const bool ex = extra.numel() > 0;
+  if (ex) {
+    CHECK_ACT(extra); CHECK_SAME(extra, out); CHECK_ACT(extra_gate); CHECK_SAME(extra_gate, out);
+    TORCH_CHECK(extra.is_contiguous() && extra.dim() == 2 && extra.size(0) == T && extra.size(1) == W);
+    TORCH_CHECK(extra_gate.dim() == 1 && extra_gate.size(0) == T);
+  }
   if (T == 0) return;
   seq_launch_moe_combine(out.data_ptr(), rows.data_ptr(), h.data_ptr(), rowidx.data_ptr<int>(),
-                         w.data_ptr<float>(), T, W, top, f32flag(out), cur_stream());
+                         weighted ? w.data_ptr<float>() : nullptr, ex ? extra.data_ptr() : nullptr,
+                         ex ? extra_gate.data_ptr() : nullptr, ex ? (int)extra_gate.stride(0) : 0, T, W, top,
+                         f32flag(out), cur_stream());
 }
 
 void wkv_recurrence(torch::Tensor o, torch::Tensor r, torch::Tensor k, torch::Tensor v, torch::Tensor d,
@@ -569,6 +680,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("token_shift_mix", &token_shift_mix);
   m.def("moe_route", &moe_route);
   m.def("moe_combine", &moe_combine);
+  m.def("gelu_tanh", &gelu_tanh);
+  m.def("scale_softcap", &scale_softcap);
+  m.def("scale_rows", &scale_rows);
+  m.def("latent_kv_store", &latent_kv_store);
+  m.def("attn_latent_paged", &attn_latent_paged);
   m.def("wkv_recurrence", &wkv_recurrence);
   m.def("mlstm_recurrence", &mlstm_recurrence);
   m.def("head_gate", &head_gate);

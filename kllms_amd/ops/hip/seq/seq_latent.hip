@@ -1,0 +1,434 @@
+// Latent attention: every token caches ONE row [latent c (C) | rotated key
+// part (R)] that all heads share. In the absorbed form a head's query is
+// [W_uk^T q_unrotated (C) | q_rotated (R)], its score against token j is the
+// dot product with j's cached row, and its output is the weighted sum of the
+// latents (W_uv is applied afterwards). The kernels here:
+//   latent_kv_store    query rotation in place, latent RMS norm, key-part
+//                      rotation, paged store of the cached row
+//   attn_latent_paged  sliding-window softmax attention over the paged rows
+//     - a plain kernel (any size, bf16 or fp32; the exact-mode path)
+//     - an MFMA kernel (bf16): 32 (row, head) query columns of one workgroup
+//       share each staged tile of 32 cached rows, for prompt portions,
+//       decoded tokens and mixes alike.
+// Scores, softmax weights and the running sums are fp32 everywhere.
+
+#include "seq_common.h"
+
+// ---- step input ----------------------------------------------------------------
+// grid (T, H + 1), one wave. Blocks 0..H-1: rotate the last R entries of query
+// head h (interleaved pairs, angle = float(pos) * inv_freq[i]) in place. Block
+// H: the token's down-projection row dkv [C + R] -> cache row
+// [rms(dkv[:C]) * w | rotate(dkv[C:])].
+template <typename T>
+__global__ void latent_kv_store_kernel(T* __restrict__ q, const T* __restrict__ dkv,
+                                       const float* __restrict__ w, float eps,
+                                       const int64_t* __restrict__ positions,
+                                       const float* __restrict__ inv_freq, T* __restrict__ cache,
+                                       const int64_t* __restrict__ slots, int H, int D, int R, int C,
+                                       int q_stride, int dkv_stride) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float pos = (float)positions[t];
+  if (h < H) {
+    T* row = q + (int64_t)t * q_stride + (int64_t)h * (D + R) + D;
+    for (int i = lane; i < R / 2; i += WAVE) {
+      float s, c;
+      sincosf(pos * inv_freq[i], &s, &c);
+      const float u = ldf(row + 2 * i), v = ldf(row + 2 * i + 1);
+      stf(row + 2 * i, u * c - v * s);
+      stf(row + 2 * i + 1, v * c + u * s);
+    }
+    return;
+  }
+  const T* src = dkv + (int64_t)t * dkv_stride;
+  T* dst = cache + slots[t] * (int64_t)(C + R);
+  float ss = 0.f;
+  for (int i = lane; i < C; i += WAVE) { const float x = ldf(src + i); ss += x * x; }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)C + eps);
+  for (int i = lane; i < C; i += WAVE) stf(dst + i, ldf(src + i) * r * w[i]);
+  for (int i = lane; i < R / 2; i += WAVE) {
+    float s, c;
+    sincosf(pos * inv_freq[i], &s, &c);
+    const float u = ldf(src + C + 2 * i), v = ldf(src + C + 2 * i + 1);
+    stf(dst + C + 2 * i, u * c - v * s);
+    stf(dst + C + 2 * i + 1, v * c + u * s);
+  }
+}
+
+// ---- plain attention kernel ------------------------------------------------------
+// grid (T, H), one wave per (query row, head). Visible keys lo..p in tiles of
+// 64: lane u scores key lo + tile*64 + u against the query staged in LDS, the
+// tile's weights go through LDS, then lanes own output dims and sweep the
+// tile's latent rows. Online softmax in fp32.
+#define LAT_MAX_ACC 16   // C <= 1024
+template <typename T>
+__global__ void attn_latent_paged_kernel(T* __restrict__ out, const T* __restrict__ q_abs,
+                                         const T* __restrict__ q, const T* __restrict__ cache,
+                                         const int* __restrict__ block_tables,
+                                         const int* __restrict__ token_seg,
+                                         const int64_t* __restrict__ positions, const T* __restrict__ gate,
+                                         float scale, int mask_size, int H, int D, int R, int C, int BS,
+                                         int bt_stride, int64_t qa_stride_t, int64_t qa_stride_h, int q_stride,
+                                         int gate_stride) {
+  extern __shared__ float lds[];       // query [C + R] | weights [64] | cache row index [64] (as int)
+  const int L = C + R;
+  float* qs = lds;
+  float* ps = lds + L;
+  int* rows = (int*)(ps + WAVE);
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int p = (int)positions[t];
+  const int lo = mask_size > 0 ? max(0, p - mask_size + 1) : 0;
+  const int total = p - lo + 1;
+  const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
+  const T* qa = q_abs + t * qa_stride_t + h * qa_stride_h;
+  const T* qr = q + (int64_t)t * q_stride + (int64_t)h * (D + R) + D;
+  for (int i = lane; i < C; i += WAVE) qs[i] = ldf(qa + i) * scale;
+  for (int i = lane; i < R; i += WAVE) qs[C + i] = ldf(qr + i) * scale;
+  __syncthreads();
+
+  float acc[LAT_MAX_ACC];
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_ACC; ++i) acc[i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  for (int base = 0; base < total; base += WAVE) {
+    const int u = base + lane;
+    float s = -INFINITY;
+    int row = -1;
+    if (u < total) {
+      const int j = lo + u;
+      row = bt[j / BS] * BS + (j % BS);
+      const T* kr = cache + (int64_t)row * L;
+      float d = 0.f;
+      for (int i = 0; i < L; ++i) d += qs[i] * ldf(kr + i);
+      s = d;
+    }
+    const float m_new = fmaxf(m, wave_max(s));
+    const float w = u < total ? expf(s - m_new) : 0.f;
+    const float corr = expf(m - m_new);        // m = -inf on the first tile -> 0
+    l = l * corr + wave_sum(w);
+    m = m_new;
+    ps[lane] = w;
+    rows[lane] = row;
+    __syncthreads();
+    const int n = min(WAVE, total - base);
+#pragma unroll
+    for (int i = 0; i < LAT_MAX_ACC; ++i) acc[i] *= corr;
+    for (int jj = 0; jj < n; ++jj) {
+      const float pw = ps[jj];
+      const T* vr = cache + (int64_t)rows[jj] * L;
+#pragma unroll
+      for (int i = 0; i < LAT_MAX_ACC; ++i) {
+        const int d = lane + i * WAVE;
+        if (d < C) acc[i] += pw * ldf(vr + d);
+      }
+    }
+    __syncthreads();
+  }
+  float gsc = 1.0f / l;
+  if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
+  T* orow = out + ((int64_t)t * H + h) * C;
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_ACC; ++i) {
+    const int d = lane + i * WAVE;
+    if (d < C) stf(orow + d, acc[i] * gsc);
+  }
+}
+
+// ---- MFMA attention kernel (bf16) ---------------------------------------------------
+// v_mfma_f32_32x32x16_bf16 fragment maps:
+//   A[i][k]: lane l holds i = l&31, k = (l>>5)*8 + j   (j = 0..7)
+//   B[k][j]: lane l holds j = l&31, k = (l>>5)*8 + jj
+//   C[i][j]: lane l holds j = l&31, i = (r&3) + 8*(r>>2) + 4*(l>>5)  (r = 0..15)
+//
+// A workgroup of 4 waves serves one tile of `tile_rows` consecutive packed
+// rows x `hb` heads = up to 32 query columns (column c = row c / hb, head
+// h0 + c % hb). Rows of a tile that belong to different sequences are served
+// in turn (one pass over the keys per sequence present in the tile; columns of
+// other sequences are masked out of the pass).
+//
+// Per tile of 32 keys:
+//   all threads stage the 32 cached rows [32][Lp] (zero-padded to a multiple
+//   of 16 dims) in LDS;
+//   S^T[key][col] = rows x query^T: the 16-dim slices of the dot product are
+//   dealt round-robin to the waves, each writes its partial S^T to LDS and
+//   every wave sums the four partials in the same order (so all waves hold
+//   identical scores);
+//   mask, scale, online softmax: a column's 32 scores sit in one lane pair
+//   (l, l ^ 32), the rest is lane-local;
+//   O^T[d][col] += latent^T x P: the 32-dim output tiles are dealt
+//   round-robin to the waves. P enters the matrix unit as a sum of two bf16
+//   parts (the rounding of p and the rounding of what that left), so the
+//   weights keep 16 bits of mantissa; the latent fragments are read from the
+//   staged rows by columns.
+typedef __bf16 lat_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float lat_f32x16 __attribute__((ext_vector_type(16)));
+
+#define LAT_WAVES 4
+#define LAT_KT 32            // keys per tile
+#define LAT_MAX_SL 9         // 16-dim slices per wave: C + R <= 576
+#define LAT_MAX_DT 4         // 32-dim output tiles per wave: C <= 512
+#define LAT_PAD 8            // bf16 elements of padding per staged row
+
+__device__ __forceinline__ int lat_acc_row(int r, int half) { return (r & 3) + 8 * (r >> 2) + 4 * half; }
+
+__global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
+    bfraw* __restrict__ out, const bfraw* __restrict__ q_abs, const bfraw* __restrict__ q,
+    const bfraw* __restrict__ cache, const int* __restrict__ block_tables, const int* __restrict__ token_seg,
+    const int64_t* __restrict__ positions, const bfraw* __restrict__ gate, float scale, int mask_size, int T_,
+    int H, int D, int R, int C, int BS, int bt_stride, int64_t qa_stride_t, int64_t qa_stride_h, int q_stride,
+    int gate_stride, int tile_rows, int hb, int vec) {
+  extern __shared__ __align__(16) unsigned char lat_smem[];
+  const int L = C + R;
+  const int Lp = (L + 15) / 16 * 16;
+  const int kstride = Lp + LAT_PAD;                       // staged row stride in elements
+  bfraw* k_lds = reinterpret_cast<bfraw*>(lat_smem);                                   // [32][kstride]
+  float* s_lds = reinterpret_cast<float*>(lat_smem + (size_t)LAT_KT * kstride * 2);    // [4][16][64]
+  __shared__ int row_idx[LAT_KT];
+
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const int half = lane >> 5, col = lane & 31;
+  const int row0 = blockIdx.x * tile_rows;
+  const int h0 = blockIdx.y * hb;
+  const int nrows = min(tile_rows, T_ - row0);
+  // this lane's query column
+  const int crow = col / hb, chead = h0 + col % hb;
+  const bool cvalid = crow < nrows && chead < H;
+  const int ct = row0 + (cvalid ? crow : 0);
+  const int cpos = (int)positions[ct];
+  const int cseg = token_seg[ct];
+  const int clo = mask_size > 0 ? max(0, cpos - mask_size + 1) : 0;
+
+  // query fragments (B operand) of this wave's slices: dims s*16 + half*8 + jj
+  const int nslice = Lp / 16;
+  lat_bf16x8 q_frag[LAT_MAX_SL];
+  {
+    const bfraw* qa = q_abs + ct * qa_stride_t + (cvalid ? chead : 0) * qa_stride_h;
+    const bfraw* qr = q + (int64_t)ct * q_stride + (int64_t)(cvalid ? chead : 0) * (D + R) + D;
+#pragma unroll
+    for (int i = 0; i < LAT_MAX_SL; ++i) {
+      const int s = wave + i * LAT_WAVES;
+      __attribute__((aligned(16))) bfraw e[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; ++jj) {
+        const int d = s * 16 + half * 8 + jj;
+        e[jj] = (s < nslice && cvalid && d < L) ? (d < C ? qa[d] : qr[d - C]) : (bfraw)0;
+      }
+      q_frag[i] = *reinterpret_cast<lat_bf16x8*>(e);
+    }
+  }
+
+  const int ndt = (C + 31) / 32;
+  lat_f32x16 o_acc[LAT_MAX_DT];
+#pragma unroll
+  for (int i = 0; i < LAT_MAX_DT; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o_acc[i][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  // one pass per sequence present in the tile (rows are packed by sequence)
+  int ra = 0;
+  while (ra < nrows) {
+    const int seg = token_seg[row0 + ra];
+    int rb = ra + 1;
+    while (rb < nrows && token_seg[row0 + rb] == seg) ++rb;
+    const int p_first = (int)positions[row0 + ra], p_last = (int)positions[row0 + rb - 1];
+    const int key_lo = mask_size > 0 ? max(0, p_first - mask_size + 1) : 0;
+    const int* bt = block_tables + (int64_t)seg * bt_stride;
+    const bool mine = cvalid && cseg == seg && crow >= ra && crow < rb;
+
+    for (int kt0 = key_lo; kt0 <= p_last; kt0 += LAT_KT) {
+      const int nkeys = min(LAT_KT, p_last - kt0 + 1);
+      if (tid < LAT_KT) {
+        const int j = kt0 + min(tid, nkeys - 1);
+        row_idx[tid] = bt[j / BS] * BS + (j % BS);
+      }
+      __syncthreads();
+      // ---- stage the cached rows, zero-padded ------------------------------------
+      {
+        const int chunks = Lp / 8;
+        for (int idx = tid; idx < LAT_KT * chunks; idx += WAVE * LAT_WAVES) {
+          const int key = idx / chunks, c8 = (idx - key * chunks) * 8;
+          const bfraw* src = cache + (int64_t)row_idx[key] * L + c8;
+          uint4 val = make_uint4(0, 0, 0, 0);
+          if (key < nkeys) {
+            if (vec && c8 + 8 <= L) {
+              val = *reinterpret_cast<const uint4*>(src);
+            } else {
+              __attribute__((aligned(16))) bfraw e[8];
+#pragma unroll
+              for (int jj = 0; jj < 8; ++jj) e[jj] = c8 + jj < L ? src[jj] : (bfraw)0;
+              val = *reinterpret_cast<uint4*>(e);
+            }
+          }
+          *reinterpret_cast<uint4*>(k_lds + key * kstride + c8) = val;
+        }
+      }
+      __syncthreads();
+      // ---- partial S^T over this wave's slices ---------------------------------
+      {
+        lat_f32x16 s_acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_acc[r] = 0.f;
+#pragma unroll
+        for (int i = 0; i < LAT_MAX_SL; ++i) {
+          const int s = wave + i * LAT_WAVES;
+          if (s < nslice) {
+            const lat_bf16x8 a = *reinterpret_cast<const lat_bf16x8*>(k_lds + col * kstride + s * 16 + half * 8);
+            s_acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q_frag[i], s_acc, 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s_lds[(wave * 16 + r) * WAVE + lane] = s_acc[r];
+      }
+      __syncthreads();
+      float sv[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float a = s_lds[r * WAVE + lane];
+#pragma unroll
+        for (int w2 = 1; w2 < LAT_WAVES; ++w2) a += s_lds[(w2 * 16 + r) * WAVE + lane];
+        const int kk = lat_acc_row(r, half);
+        const int key = kt0 + kk;
+        const bool ok = mine && kk < nkeys && key <= cpos && key >= clo;
+        sv[r] = ok ? a * scale : -INFINITY;
+      }
+      // ---- online softmax; a column's scores sit in lanes l and l ^ 32 -----------
+      float tmax = sv[0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sv[r]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+      const float m_new = fmaxf(m_run, tmax);
+      const float alpha = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);   // m_new = -inf only with m_run = -inf
+      m_run = m_new;
+      float p[16], psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        p[r] = (sv[r] == -INFINITY) ? 0.f : expf(sv[r] - m_new);
+        psum += p[r];
+      }
+      l_run = l_run * alpha + psum;
+#pragma unroll
+      for (int i = 0; i < LAT_MAX_DT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+      // ---- P as two bf16 parts, repacked into B fragments --------------------------
+      // B[k][j]: lane (j, hf) needs keys kt*16 + hf*8 + 0..7 of column j. Lane
+      // (j, half) holds keys lat_acc_row(r, half): r = 4g + i -> key 8g + 4*half + i.
+      // Fragment kt of lane (j, hf) = keys 16kt + 8hf + {0..3} from lane (j, 0),
+      // regs 4(2kt + hf) + {0..3}, and {4..7} from lane (j, 1), the same regs.
+      uint32_t hi2[8], lo2[8];
+#pragma unroll
+      for (int pr = 0; pr < 8; ++pr) {
+        const uint32_t h0b = bf_bits(p[2 * pr]), h1b = bf_bits(p[2 * pr + 1]);
+        union { uint32_t u; float f; } c0, c1;
+        c0.u = h0b << 16; c1.u = h1b << 16;
+        hi2[pr] = h0b | (h1b << 16);
+        lo2[pr] = bf_bits(p[2 * pr] - c0.f) | (bf_bits(p[2 * pr + 1] - c1.f) << 16);
+      }
+      lat_bf16x8 pf_hi[2], pf_lo[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        // group g = 2kt + hf: words 2g, 2g+1 of the lane with half 0, then of the lane with half 1
+        __attribute__((aligned(16))) uint32_t wh[4], wl[4];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          const int g = 2 * kt + hf;
+          // what the partner lane (other half) holds for group g
+          const uint32_t oh0 = __shfl_xor(hi2[2 * g], 32), oh1 = __shfl_xor(hi2[2 * g + 1], 32);
+          const uint32_t ol0 = __shfl_xor(lo2[2 * g], 32), ol1 = __shfl_xor(lo2[2 * g + 1], 32);
+          if (hf == half) {
+            // this lane builds its own fragment from group g: keys 0..3 from half 0, 4..7 from half 1
+            wh[0] = half == 0 ? hi2[2 * g] : oh0;  wh[1] = half == 0 ? hi2[2 * g + 1] : oh1;
+            wh[2] = half == 0 ? oh0 : hi2[2 * g];  wh[3] = half == 0 ? oh1 : hi2[2 * g + 1];
+            wl[0] = half == 0 ? lo2[2 * g] : ol0;  wl[1] = half == 0 ? lo2[2 * g + 1] : ol1;
+            wl[2] = half == 0 ? ol0 : lo2[2 * g];  wl[3] = half == 0 ? ol1 : lo2[2 * g + 1];
+          }
+        }
+        pf_hi[kt] = *reinterpret_cast<lat_bf16x8*>(wh);
+        pf_lo[kt] = *reinterpret_cast<lat_bf16x8*>(wl);
+      }
+      // ---- O^T += latent^T x P over this wave's output tiles ------------------------
+#pragma unroll
+      for (int i = 0; i < LAT_MAX_DT; ++i) {
+        const int dt = wave + i * LAT_WAVES;
+        if (dt < ndt) {
+          const int d = dt * 32 + col;            // < Lp: columns beyond C hold the key part or zeros, never stored
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt) {
+            __attribute__((aligned(16))) bfraw e[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) e[j] = k_lds[(kt * 16 + half * 8 + j) * kstride + min(d, Lp - 1)];
+            const lat_bf16x8 a = *reinterpret_cast<lat_bf16x8*>(e);
+            o_acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf_hi[kt], o_acc[i], 0, 0, 0);
+            o_acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf_lo[kt], o_acc[i], 0, 0, 0);
+          }
+        }
+      }
+      __syncthreads();
+    }
+    ra = rb;
+  }
+
+  // ---- epilogue: the column's two half sums, 1/l, gate, store ------------------------
+  l_run += __shfl_xor(l_run, 32);
+  if (cvalid) {
+    float gsc = l_run > 0.f ? 1.0f / l_run : 0.f;
+    if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)ct * gate_stride + chead));
+    bfraw* orow = out + ((int64_t)ct * H + chead) * C;
+#pragma unroll
+    for (int i = 0; i < LAT_MAX_DT; ++i) {
+      const int dt = wave + i * LAT_WAVES;
+      if (dt < ndt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int d = dt * 32 + lat_acc_row(r, half);
+          if (d < C) stf(orow + d, o_acc[i][r] * gsc);
+        }
+      }
+    }
+  }
+}
+
+#define DISPATCH_T(is_f32, ...)                                  \
+  if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
+
+extern "C" void seq_launch_latent_kv_store(void* q, const void* dkv, const float* w, float eps,
+                                           const int64_t* positions, const float* inv_freq, void* cache,
+                                           const int64_t* slots, int T_, int H, int D, int R, int C,
+                                           int q_stride, int dkv_stride, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(latent_kv_store_kernel<T>, dim3(T_, H + 1), dim3(WAVE), 0, st, (T*)q,
+                                        (const T*)dkv, w, eps, positions, inv_freq, (T*)cache, slots, H, D, R, C,
+                                        q_stride, dkv_stride);)
+}
+
+// tile_rows: rows per workgroup of the MFMA kernel (0 = as many as fit 32
+// columns); use_mfma 0 forces the plain kernel.
+extern "C" void seq_launch_attn_latent_paged(void* out, const void* q_abs, const void* q, const void* cache,
+                                             const int* block_tables, const int* token_seg,
+                                             const int64_t* positions, const void* gate, float scale,
+                                             int mask_size, int T_, int H, int D, int R, int C, int BS,
+                                             int bt_stride, int64_t qa_stride_t, int64_t qa_stride_h,
+                                             int q_stride, int gate_stride, int tile_rows, int use_mfma,
+                                             int is_f32, hipStream_t st) {
+  const int L = C + R;
+  if (use_mfma && !is_f32 && L <= 16 * LAT_WAVES * LAT_MAX_SL && C <= 32 * LAT_WAVES * LAT_MAX_DT) {
+    int hb = 1;
+    while (hb < H && hb < 32) hb <<= 1;                  // heads per tile: a power of two <= 32
+    const int max_rows = 32 / hb;
+    const int tr = tile_rows > 0 && tile_rows < max_rows ? tile_rows : max_rows;
+    const int Lp = (L + 15) / 16 * 16;
+    const size_t lds = (size_t)LAT_KT * (Lp + LAT_PAD) * 2 + (size_t)LAT_WAVES * 16 * WAVE * 4;
+    const int vec = (L % 8 == 0 && aligned16(cache)) ? 1 : 0;
+    hipLaunchKernelGGL(attn_latent_mfma_kernel, dim3((T_ + tr - 1) / tr, (H + hb - 1) / hb),
+                       dim3(WAVE * LAT_WAVES), lds, st, (bfraw*)out, (const bfraw*)q_abs, (const bfraw*)q,
+                       (const bfraw*)cache, block_tables, token_seg, positions, (const bfraw*)gate, scale,
+                       mask_size, T_, H, D, R, C, BS, bt_stride, qa_stride_t, qa_stride_h, q_stride, gate_stride,
+                       tr, hb, vec);
+    return;
+  }
+  const size_t lds = (size_t)(L + 2 * WAVE) * sizeof(float);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_latent_paged_kernel<T>, dim3(T_, H), dim3(WAVE), lds, st, (T*)out,
+                                        (const T*)q_abs, (const T*)q, (const T*)cache, block_tables, token_seg,
+                                        positions, (const T*)gate, scale, mask_size, H, D, R, C, BS, bt_stride,
+                                        qa_stride_t, qa_stride_h, q_stride, gate_stride);)
+}

@@ -4,19 +4,25 @@
 
 #include "seq_common.h"
 
-// out[t] = rmsnorm(table[ids[t]]) * w   (fp32 residual stream)
+// out[t] = rmsnorm(table[ids[t]] (+ pos_table[positions[t]])) * w   (fp32 residual stream)
 template <typename T>
 __global__ void embed_rmsnorm_kernel(float* __restrict__ out, const int64_t* __restrict__ ids,
                                      const T* __restrict__ table, const float* __restrict__ w,
+                                     const T* __restrict__ pos_table, const int64_t* __restrict__ positions,
                                      int W, float eps) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const T* row = table + (int64_t)ids[t] * W;
+  const T* prow = pos_table != nullptr ? pos_table + positions[t] * W : nullptr;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) { float v = ldf(row + i); ss += v * v; }
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float v = ldf(row + i) + (prow != nullptr ? ldf(prow + i) : 0.f);
+    ss += v * v;
+  }
   ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)W + eps);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) out[(int64_t)t * W + i] = ldf(row + i) * r * w[i];
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    out[(int64_t)t * W + i] = (ldf(row + i) + (prow != nullptr ? ldf(prow + i) : 0.f)) * r * w[i];
 }
 
 // out[t] = rmsnorm(x[t]) * w, x fp32, out in the activation type
@@ -37,6 +43,8 @@ __global__ void rmsnorm_cast_kernel(T* __restrict__ out, const float* __restrict
 //   y = (rms(a) wa + rms(b) wb) / 2          (two branches, DUAL)
 //   x += rms(y) * w_post                     (fp32 residual, in place)
 //   out = rms(x) * w_next                    (next sublayer's input; optional)
+//   out = x                                  (w_next == nullptr, out != nullptr: the
+//                                             stream itself in the activation type)
 // y is staged in dynamic LDS (W floats).
 template <typename T, bool DUAL>
 __global__ void sandwich_residual_kernel(float* __restrict__ x, const T* __restrict__ a,
@@ -75,7 +83,11 @@ __global__ void sandwich_residual_kernel(float* __restrict__ x, const T* __restr
     float v = x[base + i] + ybuf[i] * ry * w_post[i];
     x[base + i] = v; ybuf[i] = v; ssx += v * v;
   }
-  if (w_next == nullptr) return;
+  if (out == nullptr) return;
+  if (w_next == nullptr) {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + base + i, ybuf[i]);
+    return;
+  }
   ssx = block_sum(ssx, scratch);
   const float rx = 1.0f / sqrtf(ssx * invW + eps);
   for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + base + i, ybuf[i] * rx * w_next[i]);
@@ -131,7 +143,11 @@ __global__ void sandwich_residual_v8_kernel(float* __restrict__ x, const T* __re
     st8(x + base + i, va);
     st8(ybuf + i, va);
   }
-  if (w_next == nullptr) return;
+  if (out == nullptr) return;
+  if (w_next == nullptr) {
+    for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) { ld8(ybuf + i, va); st8(out + base + i, va); }
+    return;
+  }
   ssx = block_sum(ssx, scratch);
   const float rx = 1.0f / sqrtf(ssx * invW + eps);
   for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
@@ -259,14 +275,71 @@ __global__ void clamped_glu_v8_kernel(T* __restrict__ out, const T* __restrict__
   }
 }
 
+// tanh-form gelu: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+__device__ __forceinline__ float gelu_tanh_exact(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void gelu_tanh_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t n, int cols, int stride) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / cols, c = i - r * cols;
+    stf(out + i, gelu_tanh_exact(ldf(x + r * stride + c)));
+  }
+}
+
+template <typename T>
+__global__ void gelu_tanh_v8_kernel(T* __restrict__ out, const T* __restrict__ x, int64_t n8, int cols8,
+                                    int stride) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / cols8, c = (i - r * cols8) * 8;
+    float v[8];
+    ld8(x + r * stride + c, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = gelu_tanh_exact(v[e]);
+    st8(out + i * 8, v);
+  }
+}
+
+// z <- z * scale, then cap * tanh(z / cap) when cap > 0 (fp32 logits, in place)
+__global__ void scale_softcap_kernel(float* __restrict__ z, int64_t n, float scale, float cap) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const float v = z[i] * scale;
+    z[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+  }
+}
+
 #define DISPATCH_T(is_f32, ...)                                  \
   if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
 
 extern "C" void seq_launch_embed_rmsnorm(float* out, const int64_t* ids, const void* table,
-                                         const float* w, int T_, int W, float eps, int is_f32,
-                                         hipStream_t st) {
+                                         const float* w, const void* pos_table, const int64_t* positions,
+                                         int T_, int W, float eps, int is_f32, hipStream_t st) {
   DISPATCH_T(is_f32, hipLaunchKernelGGL(embed_rmsnorm_kernel<T>, dim3(T_), dim3(256), 0, st, out, ids,
-                                        (const T*)table, w, W, eps);)
+                                        (const T*)table, w, (const T*)pos_table, positions, W, eps);)
+}
+
+extern "C" void seq_launch_gelu_tanh(void* out, const void* x, int64_t rows, int cols, int stride, int is_f32,
+                                     hipStream_t st) {
+  if (cols % 8 == 0 && stride % 8 == 0 && aligned16(out) && aligned16(x)) {
+    const int64_t n8 = rows * cols / 8;
+    const int g8 = (int)((n8 + 255) / 256 < 16384 ? (n8 + 255) / 256 : 16384);
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(gelu_tanh_v8_kernel<T>, dim3(g8), dim3(256), 0, st, (T*)out,
+                                          (const T*)x, n8, cols / 8, stride);)
+    return;
+  }
+  const int64_t n = rows * cols;
+  const int grid = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(gelu_tanh_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out, (const T*)x,
+                                        n, cols, stride);)
+}
+
+extern "C" void seq_launch_scale_softcap(float* z, int64_t n, float scale, float cap, hipStream_t st) {
+  const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  hipLaunchKernelGGL(scale_softcap_kernel, dim3(grid), dim3(256), 0, st, z, n, scale, cap);
 }
 
 extern "C" void seq_launch_rmsnorm_cast(void* out, const float* x, const float* w, int T_, int W,

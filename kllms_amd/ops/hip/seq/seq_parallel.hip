@@ -275,7 +275,8 @@ __global__ void __launch_bounds__(256) moe_route_kernel(int* __restrict__ idx, f
                                                         const T* __restrict__ h,
                                                         const float* __restrict__ router,
                                                         const float* __restrict__ corr, int N, int W, int top,
-                                                        int gc, int gk, int E, int T_, int vec) {
+                                                        int gc, int gk, int E, int T_, int vec,
+                                                        int score_kind, int renorm) {
   __shared__ float cs[ROUTE_MAX_N], ss[ROUTE_MAX_N], gmax[ROUTE_MAX_N], zs[ROUTE_MAX_N];
   __shared__ int ok[ROUTE_MAX_N];
   const int64_t t = blockIdx.x;
@@ -305,14 +306,19 @@ __global__ void __launch_bounds__(256) moe_route_kernel(int* __restrict__ idx, f
   }
   __syncthreads();
   const int per = N / gc;
-  if (wave == 0) {
+  if (wave == 0 && score_kind == 0) {          // softmax over the outputs
     float mx = -INFINITY;
     for (int e = lane; e < N; e += WAVE) mx = fmaxf(mx, zs[e]);
     mx = wave_max(mx);
     float sum = 0.f;
     for (int e = lane; e < N; e += WAVE) { const float p = expf(zs[e] - mx); ss[e] = p; sum += p; }
     sum = wave_sum(sum);
-    for (int e = lane; e < N; e += WAVE) { ss[e] /= sum; cs[e] = ss[e] + corr[e]; }
+    for (int e = lane; e < N; e += WAVE) { ss[e] /= sum; cs[e] = ss[e] + (corr != nullptr ? corr[e] : 0.f); }
+  } else if (wave == 0) {                      // sigmoid of each output
+    for (int e = lane; e < N; e += WAVE) {
+      ss[e] = sigmoid_exact(zs[e]);
+      cs[e] = ss[e] + (corr != nullptr ? corr[e] : 0.f);
+    }
   }
   __syncthreads();
   if (wave == 0) {
@@ -359,21 +365,52 @@ __global__ void __launch_bounds__(256) moe_route_kernel(int* __restrict__ idx, f
     }
     __syncthreads();
   }
-  if (wave == 0 && lane < top) wout[t * top + lane] = mine / (wsum + 1e-20f);
+  if (wave == 0 && lane < top) wout[t * top + lane] = renorm ? mine / (wsum + 1e-20f) : mine;
 }
 
 // ---- combine: out[t] = sum_j w[t,j] * (rowidx[t,j] >= 0 ? rows[rowidx[t,j]] : h[t]) ------
+// w == nullptr: unweighted. extra != nullptr: + sigmoid(extra_gate[t]) * extra[t].
 template <typename T>
 __global__ void moe_combine_kernel(T* __restrict__ out, const T* __restrict__ rows, const T* __restrict__ h,
-                                   const int* __restrict__ rowidx, const float* __restrict__ w, int W, int top) {
+                                   const int* __restrict__ rowidx, const float* __restrict__ w,
+                                   const T* __restrict__ extra, const T* __restrict__ extra_gate,
+                                   int gate_stride, int W, int top) {
   const int64_t t = blockIdx.x;
+  const float eg = extra != nullptr ? sigmoid_exact(ldf(extra_gate + t * gate_stride)) : 0.f;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float acc = 0.f;
     for (int j = 0; j < top; ++j) {
       const int r = rowidx[t * top + j];
-      acc += w[t * top + j] * (r >= 0 ? ldf(rows + (int64_t)r * W + i) : ldf(h + t * W + i));
+      const float v = r >= 0 ? ldf(rows + (int64_t)r * W + i) : ldf(h + t * W + i);
+      acc += w != nullptr ? w[t * top + j] * v : v;
     }
+    if (extra != nullptr) acc += eg * ldf(extra + t * W + i);
     stf(out + t * W + i, acc);
+  }
+}
+
+// ---- out[i] = h[src_row[i]] * scale[i]: expert inputs that carry their routing weight ------
+template <typename T>
+__global__ void scale_rows_kernel(T* __restrict__ out, const T* __restrict__ h, const int* __restrict__ src_row,
+                                  const float* __restrict__ scale, int W) {
+  const int64_t r = blockIdx.x;
+  const T* src = h + (int64_t)src_row[r] * W;
+  const float sc = scale[r];
+  for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + r * W + i, ldf(src + i) * sc);
+}
+
+template <typename T>
+__global__ void scale_rows_v8_kernel(T* __restrict__ out, const T* __restrict__ h,
+                                     const int* __restrict__ src_row, const float* __restrict__ scale, int W) {
+  const int64_t r = blockIdx.x;
+  const T* src = h + (int64_t)src_row[r] * W;
+  const float sc = scale[r];
+  for (int i = threadIdx.x * 8; i < W; i += blockDim.x * 8) {
+    float v[8];
+    ld8(src + i, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= sc;
+    st8(out + r * W + i, v);
   }
 }
 
@@ -452,15 +489,31 @@ extern "C" void seq_launch_token_shift_mix(void* act, float* f32, const void* h,
 
 extern "C" void seq_launch_moe_route(int* idx, float* w, int* rowidx, const float* z, const void* h,
                                      const float* router, const float* corr, int T_, int N, int W, int top,
-                                     int gc, int gk, int E, int is_f32, hipStream_t st) {
+                                     int gc, int gk, int E, int score_kind, int renorm, int is_f32,
+                                     hipStream_t st) {
   const int vec = (h != nullptr && W % 8 == 0 && aligned16(h) && aligned16(router)) ? 1 : 0;
   const int threads = h != nullptr ? 256 : WAVE;
   DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_route_kernel<T>, dim3(T_), dim3(threads), 0, st, idx, w, rowidx, z,
-                                        (const T*)h, router, corr, N, W, top, gc, gk, E, T_, vec);)
+                                        (const T*)h, router, corr, N, W, top, gc, gk, E, T_, vec, score_kind,
+                                        renorm);)
 }
 
 extern "C" void seq_launch_moe_combine(void* out, const void* rows, const void* h, const int* rowidx,
-                                       const float* w, int T_, int W, int top, int is_f32, hipStream_t st) {
+                                       const float* w, const void* extra, const void* extra_gate,
+                                       int gate_stride, int T_, int W, int top, int is_f32, hipStream_t st) {
   DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)out,
-                                        (const T*)rows, (const T*)h, rowidx, w, W, top);)
+                                        (const T*)rows, (const T*)h, rowidx, w, (const T*)extra,
+                                        (const T*)extra_gate, gate_stride, W, top);)
+}
+
+extern "C" void seq_launch_scale_rows(void* out, const void* h, const int* src_row, const float* scale, int n,
+                                      int W, int is_f32, hipStream_t st) {
+  if (W % 8 == 0 && aligned16(out) && aligned16(h)) {
+    const int threads = W / 8 >= 256 ? 256 : (W / 8 > 64 ? 128 : 64);
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(scale_rows_v8_kernel<T>, dim3(n), dim3(threads), 0, st, (T*)out,
+                                          (const T*)h, src_row, scale, W);)
+    return;
+  }
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(scale_rows_kernel<T>, dim3(n), dim3(row_threads(W)), 0, st, (T*)out,
+                                        (const T*)h, src_row, scale, W);)
 }

@@ -273,9 +273,12 @@ def sample(
 # recurrent state is taken as zero whatever its slot holds). A decode step is
 # the case of all segments having one row.
 
-def embed_rmsnorm(ids: torch.Tensor, table: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """fp32 residual stream: rmsnorm(table[ids]) * weight."""
+def embed_rmsnorm(ids: torch.Tensor, table: torch.Tensor, weight: torch.Tensor, eps: float,
+                  pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 residual stream: rmsnorm(table[ids] (+ pos_table[positions])) * weight."""
     x = table[ids].float()
+    if pos_table is not None:
+        x = x + pos_table[positions].float()
     return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
 
 
@@ -284,11 +287,11 @@ def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype) -
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
 
 
-def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, out_dtype=None):
+def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, out_dtype=None, cast=False):
     """x (fp32, in place) += rmsnorm(y) * w_post, where y = a, or with a second
     branch y = (rmsnorm(a) * wa + rmsnorm(b) * wb) / 2. Returns
-    rmsnorm(x) * w_next cast to out_dtype (the next sublayer's input), or None
-    when w_next is None."""
+    rmsnorm(x) * w_next cast to out_dtype (the next sublayer's input); with
+    w_next None: x itself cast to out_dtype if ``cast``, else None."""
     def n(t):
         t = t.float()
         return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)
@@ -298,7 +301,7 @@ def sandwich_residual(x, a, w_post, eps, b=None, wa=None, wb=None, w_next=None, 
         y = 0.5 * (n(a) * wa.float() + n(b) * wb.float())
     x.add_(n(y) * w_post.float())
     if w_next is None:
-        return None
+        return x.to(out_dtype) if cast else None
     return (n(x) * w_next.float()).to(out_dtype)
 
 
@@ -659,15 +662,16 @@ def gated_act(gate, up, limit: float, alpha: float, up_bias: float) -> torch.Ten
     return (g * torch.sigmoid(alpha * g) * (u + up_bias)).to(gate.dtype)
 
 
-def moe_route(z, correction, top, group_count, group_keep):
-    """z [T, N] fp32 router logits. Scores s = softmax(z); the choice is made
-    on c = s + correction among the experts of the ``group_keep`` groups (of
+def moe_route(z, correction, top, group_count, group_keep, score="softmax", renormalize=True):
+    """z [T, N] fp32 router logits. Scores s = softmax(z) over the outputs, or
+    sigmoid(z) of each; the choice is made on c = s + correction (None = no
+    correction) among the experts of the ``group_keep`` groups (of
     ``group_count`` equal runs of neighbours) whose largest c is largest;
     ties go to the lower index. Returns (idx [T, top] int32, w [T, top] fp32
-    = chosen s / (their sum + 1e-20))."""
+    = chosen s, divided by (their sum + 1e-20) if ``renormalize``)."""
     T, N = z.shape
-    s = torch.softmax(z.float(), -1)
-    c = s + correction.float()
+    s = torch.softmax(z.float(), -1) if score == "softmax" else torch.sigmoid(z.float())
+    c = s + correction.float() if correction is not None else s
     per = N // group_count
     gs = c.view(T, group_count, per).max(-1).values
     # stable descending order = ties to the lower index
@@ -677,18 +681,99 @@ def moe_route(z, correction, top, group_count, group_keep):
     cm = torch.where(gmask.repeat_interleave(per, dim=1), c, torch.full_like(c, float("-inf")))
     idx = torch.sort(cm, dim=-1, descending=True, stable=True).indices[:, :top]
     w = s.gather(1, idx)
-    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    if renormalize:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
     return idx.to(torch.int32), w
 
 
-def moe_combine(rows, h, rowidx, w, out_dtype) -> torch.Tensor:
+def moe_combine(rows, h, rowidx, w, out_dtype, extra=None, extra_gate=None) -> torch.Tensor:
     """out[t] = sum_j w[t, j] * (rows[rowidx[t, j]] if rowidx >= 0 else h[t]),
-    summed in the order j = 0, 1, ... in fp32. rows [R, W], h [T, W]."""
+    summed in the order j = 0, 1, ... in fp32 (w None = all ones); then
+    + sigmoid(extra_gate[t]) * extra[t] when given. rows [R, W], h [T, W]."""
     T, top = rowidx.shape
     out = torch.zeros(T, h.shape[1], dtype=torch.float32, device=h.device)
     hf = h.float()
     for j in range(top):
         ri = rowidx[:, j].long()
         src = torch.where((ri >= 0)[:, None], rows[ri.clamp(min=0)].float(), hf)
-        out += w[:, j:j + 1].float() * src
+        out += src if w is None else w[:, j:j + 1].float() * src
+    if extra is not None:
+        out += torch.sigmoid(extra_gate.float()).reshape(T, 1) * extra.float()
     return out.to(out_dtype)
+
+
+def scale_rows(h, src_row, scale) -> torch.Tensor:
+    """out[i] = h[src_row[i]] * scale[i] (product in fp32), in h's dtype."""
+    return (h[src_row.long()].float() * scale.float()[:, None]).to(h.dtype)
+
+
+def gelu_tanh(x) -> torch.Tensor:
+    """0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) in fp32, in x's dtype."""
+    z = x.float()
+    return (0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))).to(x.dtype)
+
+
+def scale_softcap_(z, scale: float, cap: float) -> None:
+    """fp32 logits in place: z <- z * scale, then cap * tanh(z / cap) if cap > 0."""
+    z.mul_(scale)
+    if cap > 0:
+        z.copy_(cap * torch.tanh(z / cap))
+
+
+def latent_kv_store(q, dkv, w_norm, eps, positions, inv_freq, cache, slot_mapping, nope_dim) -> None:
+    """Latent-attention step input. q [T, H, nope_dim + R]: the last R entries
+    of every head are rotated in place (interleaved pairs, angle = position *
+    inv_freq[i], fp32). dkv [T, C + R]: the first C entries are RMS-normed
+    (weight w_norm [C]) -> the latent; the last R rotated -> the shared key
+    part. cache [NB, 1, BS, C + R] takes the row [latent | rotated part] at
+    the token's flat slot."""
+    T, H, _ = q.shape
+    R2 = inv_freq.numel()
+    R = 2 * R2
+    C = dkv.shape[1] - R
+    BS = cache.shape[2]
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    cos, sin = torch.cos(ang), torch.sin(ang)
+
+    def rot(x):                        # [..., R] with leading dim T
+        xf = x.float()
+        u, v = xf[..., 0::2], xf[..., 1::2]
+        shp = (T,) + (1,) * (xf.dim() - 2) + (R2,)
+        c, s_ = cos.view(shp), sin.view(shp)
+        out = torch.empty_like(xf)
+        out[..., 0::2] = u * c - v * s_
+        out[..., 1::2] = v * c + u * s_
+        return out
+
+    q[:, :, nope_dim:] = rot(q[:, :, nope_dim:]).to(q.dtype)
+    d = dkv[:, :C].float()
+    lat = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w_norm.float()
+    row = torch.cat([lat, rot(dkv[:, C:])], -1).to(cache.dtype)
+    sl = slot_mapping.long()
+    cache[sl // BS, 0, sl % BS] = row
+
+
+def attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale, mask_size, gate,
+                      nope_dim, out_dtype=None) -> torch.Tensor:
+    """Latent attention in its absorbed form. q_abs [T, H, C]: the unrotated
+    query parts already multiplied into the latent space; q [T, H, nope_dim +
+    R]: its last R entries are the rotated query parts. cache [NB, 1, BS,
+    C + R] rows [latent | rotated key part]. Row t at position p sees keys j
+    of its own sequence with 0 <= p - j < mask_size (0 = all j <= p):
+      score = (q_abs . latent_j + q_rot . krot_j) * scale,  softmax in fp32,
+      out[t, h] = sum_j weight_j latent_j   (times sigmoid(gate[t, h]))."""
+    T, H, C = q_abs.shape
+    BS = cache.shape[2]
+    out = torch.empty(T, H, C, dtype=out_dtype or q.dtype, device=q.device)
+    pos, seg = positions.tolist(), token_seg.tolist()
+    for t in range(T):
+        p = pos[t]
+        lo = max(0, p - mask_size + 1) if mask_size > 0 else 0
+        idx = torch.arange(lo, p + 1, device=q.device)
+        rows = cache[block_tables[seg[t]].long()[idx // BS], 0, idx % BS].float()        # [n, C+R]
+        s = (q_abs[t].float() @ rows[:, :C].T + q[t, :, nope_dim:].float() @ rows[:, C:].T) * scale
+        o = torch.softmax(s, -1) @ rows[:, :C]
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float())[:, None]
+        out[t] = o.to(out.dtype)
+    return out
