@@ -135,3 +135,52 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int], layers_out
     if cap:
         z = cap * torch.tanh(z / cap)
     return z
+
+
+def random_weights(cfg: dict, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """Random float64 tensors (already rounded to bfloat16 values) under the
+    checkpoint's names for a config in config.json form."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+
+    def mat(o, i, std=None):
+        return (torch.randn(o, i, generator=g, dtype=F64) * (std if std is not None else i ** -0.5)).bfloat16().double()
+
+    def vec(n):
+        return (1.0 + 0.2 * torch.randn(n, generator=g, dtype=F64)).bfloat16().double()
+
+    w = {"embed": mat(cfg["vocab"], W, 1.0), "pos": mat(cfg.get("max_positions", 2048), W, 0.5),
+         "embed.norm": vec(W), "final.norm": vec(W), "head": mat(cfg["vocab"], W)}
+    for i, spec in enumerate(cfg["layers"]):
+        if spec.get("weights_of", i) != i:
+            continue
+        m, pre = spec["mixer"], f"l{i}."
+        H, D, R, V, C = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+        w[pre + "norm1"] = vec(W)
+        w[pre + "mix.q"] = mat(H * (D + R), W)
+        w[pre + "mix.dkv"] = mat(C + R, W)
+        w[pre + "mix.dkv.norm"] = vec(C)
+        w[pre + "mix.uk"] = mat(H * D, C)
+        w[pre + "mix.uv"] = mat(H * V, C)
+        w[pre + "mix.g"] = mat(H, W)
+        w[pre + "mix.o"] = mat(W, H * V)
+        mlp = spec.get("mlp")
+        if not mlp:
+            continue
+        w[pre + "norm2"] = vec(W)
+        if mlp["kind"] == "dense":
+            w[pre + "mlp.up"] = mat(mlp["ff"], W)
+            w[pre + "mlp.down"] = mat(W, mlp["ff"])
+            continue
+        names = [f"e{e}" for e in range(mlp["router"]["experts"])]
+        sizes = [mlp["expert"]["ff"]] * len(names)
+        if mlp.get("shared"):
+            names.append("shared")
+            sizes.append(mlp["shared"]["ff"])
+            w[pre + "mlp.shared.sg"] = mat(1, W)
+        for n, ff in zip(names, sizes):
+            w[f"{pre}mlp.{n}.gate"] = mat(ff, W)
+            w[f"{pre}mlp.{n}.up"] = mat(ff, W)
+            w[f"{pre}mlp.{n}.down"] = mat(W, ff)
+        w[pre + "mlp.router"] = mat(mlp["router"]["experts"], W, 1.5 * W ** -0.5)
+    return w
