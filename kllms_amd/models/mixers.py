@@ -427,11 +427,13 @@ class LatentAttention(nn.Module):
         ops.latent_kv_store(q, s(y, "dkv"), self.dkv_norm, self.eps, batch.positions, self.inv_freq, st.k,
                             batch.slot_mapping, D)
         q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk)                   # [H, T, C]
+        # a step of single decoded tokens: one row per workgroup, a row's keys shared out over the chip
+        single = batch.mode == "decode" or (batch.host_segs is not None
+                                            and all(n == 1 for _, n in batch.host_segs))
         lat = ops.attn_latent_paged(q_abs.transpose(0, 1), q, st.k, batch.block_tables, batch.token_seg,
                                     batch.positions, sp.scale, sp.mask_size,
                                     s(y, "g") if sp.head_gate else None, D,
-                                    tile_rows=1 if batch.host_segs is not None
-                                    and all(n == 1 for _, n in batch.host_segs) else 0)       # [T, H, C]
+                                    tile_rows=1 if single else 0)                 # [T, H, C]
         att = torch.empty((T, H * V), dtype=y.dtype, device=y.device)
         torch.bmm(lat.transpose(0, 1), self.uv.transpose(1, 2), out=att.view(T, H, V).transpose(0, 1))
         return F.linear(att, self.o_proj)
@@ -622,9 +624,7 @@ class RoutedExperts(nn.Module):
         if dense:
             if on_input:
                 # expert e reads w[t, e] h[t] where it was chosen (zero rows elsewhere; they are never read back)
-                wsel = torch.zeros((T, E), dtype=torch.float32, device=h.device).scatter_(1, idx.long(), w)
-                src = torch.arange(T, dtype=torch.int32, device=h.device).repeat(E)
-                xin = ops.scale_rows(h, src, wsel.t().reshape(-1)).view(E, T, W)
+                xin = ops.moe_spread_rows(h, idx, w, E)
             else:
                 xin = h.unsqueeze(0).expand(E, T, W)
             gu = torch.bmm(xin, self.w_gate_up.transpose(1, 2)).view(E * T, 2 * sp.ff)

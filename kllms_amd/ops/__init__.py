@@ -568,6 +568,17 @@ def scale_rows(h, src_row, scale):
     return torch_ref.scale_rows(h, src_row, scale)
 
 
+def moe_spread_rows(h, idx, w, experts: int):
+    """[experts, T, W] inputs of the all-experts form when the routing weight
+    sits on the expert's input: w[t, j] * h[t] for row t's j-th choice, zero
+    rows for the experts a row did not choose."""
+    if _gpu(h):
+        out = torch.empty((experts, h.shape[0], h.shape[1]), dtype=h.dtype, device=h.device)
+        _seq().moe_spread_rows(out, h, idx, w)
+        return out
+    return torch_ref.moe_spread_rows(h, idx, w, experts)
+
+
 def gelu_tanh(x):
     """Tanh-form gelu of a [T, C] row view, in x's dtype."""
     if _gpu(x):
@@ -596,19 +607,34 @@ def latent_kv_store(q, dkv, w_norm, eps, positions, inv_freq, cache, slot_mappin
 
 
 def attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale, mask_size, gate, nope_dim,
-                      tile_rows: int = 0, use_mfma: bool = True):
+                      tile_rows: int = 0, use_mfma: bool = True, key_splits: int = 0):
     """Sliding-window softmax attention over the paged latent cache in the
     absorbed form (one shared key/value row per token for all heads):
     returns the heads' weighted latent sums [T, H, C], gated per head.
     GPU: bf16 rows go through the matrix-unit kernel when the sizes fit it
     (``tile_rows`` = query rows per workgroup, 0 = as many as fit 32 (row,
     head) columns; 1 suits steps of single decoded tokens), fp32 rows and
-    other sizes through the plain kernel."""
+    other sizes through the plain kernel. ``key_splits`` (with tile_rows 1):
+    workgroups that share one row's keys, merged by a second kernel; 0 = as
+    many as fill the chip for this step (few rows, long windows), -1 = none."""
     if _gpu(q):
-        out = torch.empty((q.shape[0], q.shape[1], q_abs.shape[2]), dtype=q.dtype, device=q.device)
+        T, H, C = q.shape[0], q.shape[1], q_abs.shape[2]
+        out = torch.empty((T, H, C), dtype=q.dtype, device=q.device)
+        ns = 1
+        if tile_rows == 1 and use_mfma and q.dtype == torch.bfloat16 and key_splits >= 0:
+            # an upper bound of a row's 32-key tiles, from the window or the block table's width
+            reach = mask_size if mask_size > 0 else block_tables.shape[1] * cache.shape[2]
+            reach = min(reach, block_tables.shape[1] * cache.shape[2])
+            tiles = max(1, (reach + 31) // 32)
+            groups = T * ((H + 31) // 32)
+            ns = key_splits or max(1, min((tiles + 1) // 2, 1024 // max(1, groups)))
+            ns = max(1, min(ns, tiles))
+        f = torch.float32
+        part_o = torch.empty((T, H, ns, C), dtype=f, device=q.device) if ns > 1 else _none(q, f)
+        part_ml = torch.empty((T, H, ns, 2), dtype=f, device=q.device) if ns > 1 else _none(q, f)
         _seq().attn_latent_paged(out, q_abs, q, cache, block_tables, token_seg, positions,
                                  gate if gate is not None else _none(q), float(scale), int(mask_size),
-                                 int(nope_dim), int(tile_rows), bool(use_mfma))
+                                 int(nope_dim), int(tile_rows), bool(use_mfma), part_o, part_ml)
         return out
     return torch_ref.attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale, mask_size,
                                        gate, nope_dim)

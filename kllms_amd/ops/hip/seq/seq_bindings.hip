@@ -13,11 +13,12 @@ void seq_launch_embed_rmsnorm(float*, const int64_t*, const void*, const float*,
 void seq_launch_gelu_tanh(void*, const void*, int64_t, int, int, int, hipStream_t);
 void seq_launch_scale_softcap(float*, int64_t, float, float, hipStream_t);
 void seq_launch_scale_rows(void*, const void*, const int*, const float*, int, int, int, hipStream_t);
+void seq_launch_moe_spread_rows(void*, const void*, const int*, const float*, int, int, int, int, int, hipStream_t);
 void seq_launch_latent_kv_store(void*, const void*, const float*, float, const int64_t*, const float*, void*,
                                 const int64_t*, int, int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_attn_latent_paged(void*, const void*, const void*, const void*, const int*, const int*,
                                   const int64_t*, const void*, float, int, int, int, int, int, int, int, int,
-                                  int64_t, int64_t, int, int, int, int, int, hipStream_t);
+                                  int64_t, int64_t, int, int, int, int, float*, float*, int, int, hipStream_t);
 void seq_launch_rmsnorm_cast(void*, const float*, const float*, int, int, float, int, hipStream_t);
 void seq_launch_sandwich_residual(float*, const void*, const void*, const float*, const float*, const float*,
                                   const float*, void*, int, int, float, int, hipStream_t);
@@ -134,6 +135,18 @@ void scale_rows(torch::Tensor out, torch::Tensor h, torch::Tensor src_row, torch
                         f32flag(out), cur_stream());
 }
 
+// out [E, T, W]: expert e's input rows, w[t, j] * h[t] where e is row t's j-th choice, else zero
+void moe_spread_rows(torch::Tensor out, torch::Tensor h, torch::Tensor idx, torch::Tensor w) {
+  CHECK_ACT(out); CHECK_ACT(h); CHECK_SAME(h, out); CHECK_I32C(idx); CHECK_F32C(w);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && out.dim() == 3 && out.is_contiguous());
+  const int E = out.size(0), T = h.size(0), W = h.size(1);
+  TORCH_CHECK(out.size(1) == T && out.size(2) == W && idx.dim() == 2 && idx.size(0) == T && w.numel() == idx.numel());
+  TORCH_CHECK((int64_t)E * T < (1LL << 31));
+  if (E * T == 0) return;
+  seq_launch_moe_spread_rows(out.data_ptr(), h.data_ptr(), idx.data_ptr<int>(), w.data_ptr<float>(), E, T, W,
+                             (int)idx.size(1), f32flag(out), cur_stream());
+}
+
 // q [T, H, D + R] row view (rotated in place), dkv [T, C + R] row view,
 // cache [NB, 1, BS, C + R] contiguous
 void latent_kv_store(torch::Tensor q, torch::Tensor dkv, torch::Tensor w, double eps, torch::Tensor positions,
@@ -159,7 +172,7 @@ void latent_kv_store(torch::Tensor q, torch::Tensor dkv, torch::Tensor w, double
 void attn_latent_paged(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q, torch::Tensor cache,
                        torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
                        torch::Tensor gate, double scale, int64_t mask_size, int64_t nope_dim, int64_t tile_rows,
-                       bool use_mfma) {
+                       bool use_mfma, torch::Tensor part_o, torch::Tensor part_ml) {
   CHECK_ACT(out); CHECK_ACT(q_abs); CHECK_SAME(q_abs, out); CHECK_ACT(q); CHECK_SAME(q, out); CHECK_ROWS3(q);
   CHECK_ACT(cache); CHECK_SAME(cache, out); CHECK_I32C(token_seg); CHECK_I64C(positions);
   TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
@@ -174,13 +187,23 @@ void attn_latent_paged(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q, 
   TORCH_CHECK((size_t)(C + R + 128) * 4 <= 64 * 1024);
   const bool g = gate.numel() > 0;
   if (g) { CHECK_ACT(gate); CHECK_SAME(gate, out); CHECK_ROWS2(gate); TORCH_CHECK(gate.size(0) == T && gate.size(1) == H); }
+  // key shares: part_o [T, H, nsplit, C], part_ml [T, H, nsplit, 2] fp32, or empty
+  int nsplit = 1;
+  if (part_o.numel() > 0) {
+    CHECK_F32C(part_o); CHECK_F32C(part_ml);
+    TORCH_CHECK(part_o.dim() == 4 && part_o.size(0) == T && part_o.size(1) == H && part_o.size(3) == C);
+    nsplit = (int)part_o.size(2);
+    TORCH_CHECK(nsplit >= 1 && nsplit <= 1024 && part_ml.numel() == (int64_t)T * H * nsplit * 2);
+  }
   if (T == 0) return;
   seq_launch_attn_latent_paged(out.data_ptr(), q_abs.data_ptr(), q.data_ptr(), cache.data_ptr(),
                                block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
                                positions.data_ptr<int64_t>(), g ? gate.data_ptr() : nullptr, (float)scale,
                                (int)mask_size, T, H, D, R, C, (int)cache.size(2), (int)block_tables.stride(0),
                                q_abs.stride(0), q_abs.stride(1), (int)q.stride(0), g ? (int)gate.stride(0) : 0,
-                               (int)tile_rows, use_mfma ? 1 : 0, f32flag(out), cur_stream());
+                               (int)tile_rows, use_mfma ? 1 : 0, nsplit > 1 ? part_o.data_ptr<float>() : nullptr,
+                               nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, nsplit, f32flag(out),
+                               cur_stream());
 }
 
 void rmsnorm_cast(torch::Tensor out, torch::Tensor x, torch::Tensor w, double eps) {
@@ -683,6 +706,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gelu_tanh", &gelu_tanh);
   m.def("scale_softcap", &scale_softcap);
   m.def("scale_rows", &scale_rows);
+  m.def("moe_spread_rows", &moe_spread_rows);
   m.def("latent_kv_store", &latent_kv_store);
   m.def("attn_latent_paged", &attn_latent_paged);
   m.def("wkv_recurrence", &wkv_recurrence);

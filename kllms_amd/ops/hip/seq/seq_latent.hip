@@ -148,7 +148,8 @@ __global__ void attn_latent_paged_kernel(T* __restrict__ out, const T* __restric
 //
 // Per tile of 32 keys:
 //   all threads stage the 32 cached rows [32][Lp] (zero-padded to a multiple
-//   of 16 dims) in LDS;
+//   of 16 dims) in LDS; the next tile's rows are already on their way from
+//   memory while the current tile is worked on;
 //   S^T[key][col] = rows x query^T: the 16-dim slices of the dot product are
 //   dealt round-robin to the waves, each writes its partial S^T to LDS and
 //   every wave sums the four partials in the same order (so all waves hold
@@ -168,25 +169,48 @@ typedef float lat_f32x16 __attribute__((ext_vector_type(16)));
 #define LAT_MAX_SL 9         // 16-dim slices per wave: C + R <= 576
 #define LAT_MAX_DT 4         // 32-dim output tiles per wave: C <= 512
 #define LAT_PAD 8            // bf16 elements of padding per staged row
+#define LAT_STAGE 9          // 16-byte chunks per staging thread: 8 threads per row, rows up to 576 wide
 
 __device__ __forceinline__ int lat_acc_row(int r, int half) { return (r & 3) + 8 * (r >> 2) + 4 * half; }
 
-__global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
+typedef float lat_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 lat_bf16x2 __attribute__((ext_vector_type(2)));
+
+// two floats -> two bf16 (round to nearest even) packed in one word, low half first
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  const lat_f32x2 v = {a, b};
+  lat_bf16x2 r = __builtin_convertvector(v, lat_bf16x2);
+  return *reinterpret_cast<uint32_t*>(&r);
+}
+
+// Workgroup barrier that orders LDS traffic only: every wave's LDS reads and
+// writes are complete (lgkmcnt 0) before it arrives, global loads in flight
+// stay in flight. The tile loop prefetches the next tile's rows into
+// registers, and a full __syncthreads would wait for them at every barrier.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xc07f);      // vmcnt 63, expcnt 7, lgkmcnt 0
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+__global__ void __launch_bounds__(WAVE * LAT_WAVES, 2) attn_latent_mfma_kernel(
     bfraw* __restrict__ out, const bfraw* __restrict__ q_abs, const bfraw* __restrict__ q,
     const bfraw* __restrict__ cache, const int* __restrict__ block_tables, const int* __restrict__ token_seg,
     const int64_t* __restrict__ positions, const bfraw* __restrict__ gate, float scale, int mask_size, int T_,
     int H, int D, int R, int C, int BS, int bt_stride, int64_t qa_stride_t, int64_t qa_stride_h, int q_stride,
-    int gate_stride, int tile_rows, int hb, int vec) {
+    int gate_stride, int tile_rows, int hb, int vec, int qvec, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
   extern __shared__ __align__(16) unsigned char lat_smem[];
   const int L = C + R;
   const int Lp = (L + 15) / 16 * 16;
   const int kstride = Lp + LAT_PAD;                       // staged row stride in elements
   bfraw* k_lds = reinterpret_cast<bfraw*>(lat_smem);                                   // [32][kstride]
   float* s_lds = reinterpret_cast<float*>(lat_smem + (size_t)LAT_KT * kstride * 2);    // [4][16][64]
-  __shared__ int row_idx[LAT_KT];
 
   const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int half = lane >> 5, col = lane & 31;
+  const int skey = tid >> 3, spart = tid & 7;              // staging role
   const int row0 = blockIdx.x * tile_rows;
   const int h0 = blockIdx.y * hb;
   const int nrows = min(tile_rows, T_ - row0);
@@ -198,23 +222,50 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
   const int cseg = token_seg[ct];
   const int clo = mask_size > 0 ? max(0, cpos - mask_size + 1) : 0;
 
-  // query fragments (B operand) of this wave's slices: dims s*16 + half*8 + jj
+  // query fragments (B operand) of this wave's slices: dims s*16 + half*8 + jj.
+  // The 32 columns' query rows [C | R] go through the (not yet used) key
+  // buffer: thread (skey, spart) loads chunks of column skey, then every lane
+  // reads its fragments back with 16-byte LDS loads.
   const int nslice = Lp / 16;
   lat_bf16x8 q_frag[LAT_MAX_SL];
   {
-    const bfraw* qa = q_abs + ct * qa_stride_t + (cvalid ? chead : 0) * qa_stride_h;
-    const bfraw* qr = q + (int64_t)ct * q_stride + (int64_t)(cvalid ? chead : 0) * (D + R) + D;
+    const int srow = skey / hb, shead = h0 + skey % hb;
+    const bool sval = srow < nrows && shead < H;
+    const int st_ = row0 + (sval ? srow : 0);
+    const bfraw* qa = q_abs + st_ * qa_stride_t + (sval ? shead : 0) * qa_stride_h;
+    const bfraw* qr = q + (int64_t)st_ * q_stride + (int64_t)(sval ? shead : 0) * (D + R) + D;
+    uint4 qst[LAT_STAGE];
+#pragma unroll
+    for (int i = 0; i < LAT_STAGE; ++i) {
+      const int c8 = (spart + 8 * i) * 8;
+      uint4 val = make_uint4(0, 0, 0, 0);
+      if (sval && c8 < L) {
+        if (qvec && c8 + 8 <= L) {                       // C % 8 == 0: a chunk lies in one of the two parts
+          val = *reinterpret_cast<const uint4*>(c8 < C ? qa + c8 : qr + (c8 - C));
+        } else {
+          __attribute__((aligned(16))) bfraw e[8];
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            const int d = c8 + jj;
+            e[jj] = d < L ? (d < C ? qa[d] : qr[d - C]) : (bfraw)0;
+          }
+          val = *reinterpret_cast<uint4*>(e);
+        }
+      }
+      qst[i] = val;
+    }
+#pragma unroll
+    for (int i = 0; i < LAT_STAGE; ++i) {
+      const int c8 = (spart + 8 * i) * 8;
+      if (c8 < Lp) *reinterpret_cast<uint4*>(k_lds + skey * kstride + c8) = qst[i];
+    }
+    __syncthreads();
 #pragma unroll
     for (int i = 0; i < LAT_MAX_SL; ++i) {
       const int s = wave + i * LAT_WAVES;
-      __attribute__((aligned(16))) bfraw e[8];
-#pragma unroll
-      for (int jj = 0; jj < 8; ++jj) {
-        const int d = s * 16 + half * 8 + jj;
-        e[jj] = (s < nslice && cvalid && d < L) ? (d < C ? qa[d] : qr[d - C]) : (bfraw)0;
-      }
-      q_frag[i] = *reinterpret_cast<lat_bf16x8*>(e);
+      if (s < nslice) q_frag[i] = *reinterpret_cast<const lat_bf16x8*>(k_lds + col * kstride + s * 16 + half * 8);
     }
+    __syncthreads();
   }
 
   const int ndt = (C + 31) / 32;
@@ -224,6 +275,7 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) o_acc[i][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
+  const float scale2 = scale * 1.4426950408889634f;
 
   // one pass per sequence present in the tile (rows are packed by sequence)
   int ra = 0;
@@ -235,35 +287,51 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
     const int key_lo = mask_size > 0 ? max(0, p_first - mask_size + 1) : 0;
     const int* bt = block_tables + (int64_t)seg * bt_stride;
     const bool mine = cvalid && cseg == seg && crow >= ra && crow < rb;
+    // gridDim.z > 1 (single-row tiles only): this workgroup takes a contiguous
+    // share of the row's key tiles and leaves an unnormalised partial result
+    int k_begin = key_lo, k_last = p_last;
+    if (gridDim.z > 1) {
+      const int ntiles = (p_last - key_lo) / LAT_KT + 1;
+      const int tps = (ntiles + gridDim.z - 1) / gridDim.z;
+      k_begin = key_lo + (int)blockIdx.z * tps * LAT_KT;
+      k_last = min(p_last, k_begin + tps * LAT_KT - 1);
+    }
 
-    for (int kt0 = key_lo; kt0 <= p_last; kt0 += LAT_KT) {
-      const int nkeys = min(LAT_KT, p_last - kt0 + 1);
-      if (tid < LAT_KT) {
-        const int j = kt0 + min(tid, nkeys - 1);
-        row_idx[tid] = bt[j / BS] * BS + (j % BS);
-      }
-      __syncthreads();
-      // ---- stage the cached rows, zero-padded ------------------------------------
-      {
-        const int chunks = Lp / 8;
-        for (int idx = tid; idx < LAT_KT * chunks; idx += WAVE * LAT_WAVES) {
-          const int key = idx / chunks, c8 = (idx - key * chunks) * 8;
-          const bfraw* src = cache + (int64_t)row_idx[key] * L + c8;
-          uint4 val = make_uint4(0, 0, 0, 0);
-          if (key < nkeys) {
-            if (vec && c8 + 8 <= L) {
-              val = *reinterpret_cast<const uint4*>(src);
-            } else {
-              __attribute__((aligned(16))) bfraw e[8];
+    // Staging: thread (skey, spart) of the 32 x 8 grid loads the 16-byte chunks
+    // spart, spart + 8, ... of cached row skey. The loads of the NEXT tile are
+    // issued before the current tile is worked on and land in LDS after it.
+    uint4 stage[LAT_STAGE];
+    auto fetch = [&](int kt0) {
+      const int nk = min(LAT_KT, k_last - kt0 + 1);
+      const int j = kt0 + min(skey, nk - 1);
+      const bfraw* src = cache + (int64_t)(bt[j / BS] * BS + (j % BS)) * L;
 #pragma unroll
-              for (int jj = 0; jj < 8; ++jj) e[jj] = c8 + jj < L ? src[jj] : (bfraw)0;
-              val = *reinterpret_cast<uint4*>(e);
-            }
+      for (int i = 0; i < LAT_STAGE; ++i) {
+        const int c8 = (spart + 8 * i) * 8;
+        uint4 val = make_uint4(0, 0, 0, 0);
+        if (skey < nk && c8 < Lp) {
+          if (vec && c8 + 8 <= L) {
+            val = *reinterpret_cast<const uint4*>(src + c8);
+          } else {
+            __attribute__((aligned(16))) bfraw e[8];
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) e[jj] = c8 + jj < L ? src[c8 + jj] : (bfraw)0;
+            val = *reinterpret_cast<uint4*>(e);
           }
-          *reinterpret_cast<uint4*>(k_lds + key * kstride + c8) = val;
         }
+        stage[i] = val;
       }
-      __syncthreads();
+    };
+    if (k_begin <= k_last) fetch(k_begin);
+    for (int kt0 = k_begin; kt0 <= k_last; kt0 += LAT_KT) {
+      const int nkeys = min(LAT_KT, k_last - kt0 + 1);
+#pragma unroll
+      for (int i = 0; i < LAT_STAGE; ++i) {
+        const int c8 = (spart + 8 * i) * 8;
+        if (c8 < Lp) *reinterpret_cast<uint4*>(k_lds + skey * kstride + c8) = stage[i];
+      }
+      lds_barrier();
+      if (kt0 + LAT_KT <= k_last) fetch(kt0 + LAT_KT);
       // ---- partial S^T over this wave's slices ---------------------------------
       {
         lat_f32x16 s_acc;
@@ -280,7 +348,7 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) s_lds[(wave * 16 + r) * WAVE + lane] = s_acc[r];
       }
-      __syncthreads();
+      lds_barrier();
       float sv[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -290,7 +358,7 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
         const int kk = lat_acc_row(r, half);
         const int key = kt0 + kk;
         const bool ok = mine && kk < nkeys && key <= cpos && key >= clo;
-        sv[r] = ok ? a * scale : -INFINITY;
+        sv[r] = ok ? a * scale2 : -INFINITY;            // scores in units of ln 2: weights are 2^(s - m)
       }
       // ---- online softmax; a column's scores sit in lanes l and l ^ 32 -----------
       float tmax = sv[0];
@@ -298,19 +366,22 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
       for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sv[r]);
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
       const float m_new = fmaxf(m_run, tmax);
-      const float alpha = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);   // m_new = -inf only with m_run = -inf
+      const float m_ref = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: every weight below is 2^-inf = 0
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
       m_run = m_new;
       float p[16], psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        p[r] = (sv[r] == -INFINITY) ? 0.f : expf(sv[r] - m_new);
+        p[r] = __builtin_amdgcn_exp2f(sv[r] - m_ref);
         psum += p[r];
       }
       l_run = l_run * alpha + psum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {           // the running maximum moved in some column
 #pragma unroll
-      for (int i = 0; i < LAT_MAX_DT; ++i)
+        for (int i = 0; i < LAT_MAX_DT; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+          for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+      }
       // ---- P as two bf16 parts, repacked into B fragments --------------------------
       // B[k][j]: lane (j, hf) needs keys kt*16 + hf*8 + 0..7 of column j. Lane
       // (j, half) holds keys lat_acc_row(r, half): r = 4g + i -> key 8g + 4*half + i.
@@ -319,11 +390,10 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
       uint32_t hi2[8], lo2[8];
 #pragma unroll
       for (int pr = 0; pr < 8; ++pr) {
-        const uint32_t h0b = bf_bits(p[2 * pr]), h1b = bf_bits(p[2 * pr + 1]);
+        hi2[pr] = pack_bf16x2(p[2 * pr], p[2 * pr + 1]);
         union { uint32_t u; float f; } c0, c1;
-        c0.u = h0b << 16; c1.u = h1b << 16;
-        hi2[pr] = h0b | (h1b << 16);
-        lo2[pr] = bf_bits(p[2 * pr] - c0.f) | (bf_bits(p[2 * pr + 1] - c1.f) << 16);
+        c0.u = hi2[pr] << 16; c1.u = hi2[pr] & 0xffff0000u;
+        lo2[pr] = pack_bf16x2(p[2 * pr] - c0.f, p[2 * pr + 1] - c1.f);
       }
       lat_bf16x8 pf_hi[2], pf_lo[2];
 #pragma unroll
@@ -364,28 +434,83 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES) attn_latent_mfma_kernel(
           }
         }
       }
-      __syncthreads();
+      lds_barrier();
     }
     ra = rb;
   }
 
   // ---- epilogue: the column's two half sums, 1/l, gate, store ------------------------
   l_run += __shfl_xor(l_run, 32);
+  if (gridDim.z > 1) {
+    // partial result of this key share: [T, H, splits, C] sums and (max, sum) in units of ln 2
+    if (cvalid) {
+      const int64_t slot = ((int64_t)ct * H + chead) * gridDim.z + blockIdx.z;
+      if (wave == 0 && half == 0) { part_ml[2 * slot] = m_run; part_ml[2 * slot + 1] = l_run; }
+      float* po = part_o + slot * C;
+#pragma unroll
+      for (int i = 0; i < LAT_MAX_DT; ++i) {
+        const int dt = wave + i * LAT_WAVES;
+        if (dt < ndt) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int d = dt * 32 + lat_acc_row(r, half);
+            if (d < C) po[d] = o_acc[i][r];
+          }
+        }
+      }
+    }
+    return;
+  }
   if (cvalid) {
     float gsc = l_run > 0.f ? 1.0f / l_run : 0.f;
     if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)ct * gate_stride + chead));
     bfraw* orow = out + ((int64_t)ct * H + chead) * C;
+    const bool ovec = C % 4 == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0;
 #pragma unroll
     for (int i = 0; i < LAT_MAX_DT; ++i) {
       const int dt = wave + i * LAT_WAVES;
       if (dt < ndt) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int d = dt * 32 + lat_acc_row(r, half);
-          if (d < C) stf(orow + d, o_acc[i][r] * gsc);
+        for (int g4 = 0; g4 < 4; ++g4) {               // regs 4 g4 .. 4 g4 + 3 hold 4 consecutive dims
+          const int d = dt * 32 + 8 * g4 + 4 * half;
+          if (ovec && d + 4 <= C) {
+            uint2 wd;
+            wd.x = pack_bf16x2(o_acc[i][4 * g4] * gsc, o_acc[i][4 * g4 + 1] * gsc);
+            wd.y = pack_bf16x2(o_acc[i][4 * g4 + 2] * gsc, o_acc[i][4 * g4 + 3] * gsc);
+            *reinterpret_cast<uint2*>(orow + d) = wd;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (d + e < C) stf(orow + d + e, o_acc[i][4 * g4 + e] * gsc);
+          }
         }
       }
     }
+  }
+}
+
+// Merge of the key shares' partial results: grid (T, H), one wave.
+__global__ void attn_latent_merge_kernel(bfraw* __restrict__ out, const float* __restrict__ part_o,
+                                         const float* __restrict__ part_ml, const bfraw* __restrict__ gate,
+                                         int H, int C, int nsplit, int gate_stride) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int64_t base = ((int64_t)t * H + h) * nsplit;
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) M = fmaxf(M, part_ml[2 * (base + z)]);
+  float Lsum = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float l = part_ml[2 * (base + z) + 1];
+    if (l > 0.f) Lsum += l * __builtin_amdgcn_exp2f(part_ml[2 * (base + z)] - M);
+  }
+  float gsc = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+  if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
+  for (int d = lane; d < C; d += WAVE) {
+    float acc = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float l = part_ml[2 * (base + z) + 1];
+      if (l > 0.f) acc += part_o[(base + z) * C + d] * __builtin_amdgcn_exp2f(part_ml[2 * (base + z)] - M);
+    }
+    stf(out + ((int64_t)t * H + h) * C + d, acc * gsc);
   }
 }
 
@@ -402,14 +527,17 @@ extern "C" void seq_launch_latent_kv_store(void* q, const void* dkv, const float
 }
 
 // tile_rows: rows per workgroup of the MFMA kernel (0 = as many as fit 32
-// columns); use_mfma 0 forces the plain kernel.
+// columns); use_mfma 0 forces the plain kernel. part_o [T, H, nsplit, C] /
+// part_ml [T, H, nsplit, 2] (fp32, optional): with single-row tiles the keys of
+// a row are shared out to nsplit workgroups and merged by a second kernel.
 extern "C" void seq_launch_attn_latent_paged(void* out, const void* q_abs, const void* q, const void* cache,
                                              const int* block_tables, const int* token_seg,
                                              const int64_t* positions, const void* gate, float scale,
                                              int mask_size, int T_, int H, int D, int R, int C, int BS,
                                              int bt_stride, int64_t qa_stride_t, int64_t qa_stride_h,
                                              int q_stride, int gate_stride, int tile_rows, int use_mfma,
-                                             int is_f32, hipStream_t st) {
+                                             float* part_o, float* part_ml, int nsplit, int is_f32,
+                                             hipStream_t st) {
   const int L = C + R;
   if (use_mfma && !is_f32 && L <= 16 * LAT_WAVES * LAT_MAX_SL && C <= 32 * LAT_WAVES * LAT_MAX_DT) {
     int hb = 1;
@@ -419,11 +547,17 @@ extern "C" void seq_launch_attn_latent_paged(void* out, const void* q_abs, const
     const int Lp = (L + 15) / 16 * 16;
     const size_t lds = (size_t)LAT_KT * (Lp + LAT_PAD) * 2 + (size_t)LAT_WAVES * 16 * WAVE * 4;
     const int vec = (L % 8 == 0 && aligned16(cache)) ? 1 : 0;
-    hipLaunchKernelGGL(attn_latent_mfma_kernel, dim3((T_ + tr - 1) / tr, (H + hb - 1) / hb),
+    const int qvec = (C % 8 == 0 && D % 8 == 0 && R % 8 == 0 && q_stride % 8 == 0 && qa_stride_t % 8 == 0 &&
+                      qa_stride_h % 8 == 0 && aligned16(q) && aligned16(q_abs)) ? 1 : 0;
+    const int ns = (tr == 1 && part_o != nullptr && nsplit > 1) ? nsplit : 1;
+    hipLaunchKernelGGL(attn_latent_mfma_kernel, dim3((T_ + tr - 1) / tr, (H + hb - 1) / hb, ns),
                        dim3(WAVE * LAT_WAVES), lds, st, (bfraw*)out, (const bfraw*)q_abs, (const bfraw*)q,
                        (const bfraw*)cache, block_tables, token_seg, positions, (const bfraw*)gate, scale,
                        mask_size, T_, H, D, R, C, BS, bt_stride, qa_stride_t, qa_stride_h, q_stride, gate_stride,
-                       tr, hb, vec);
+                       tr, hb, vec, qvec, part_o, part_ml);
+    if (ns > 1)
+      hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(T_, H), dim3(WAVE), 0, st, (bfraw*)out, part_o, part_ml,
+                         (const bfraw*)gate, H, C, ns, gate_stride);
     return;
   }
   const size_t lds = (size_t)(L + 2 * WAVE) * sizeof(float);

@@ -399,6 +399,20 @@ __global__ void scale_rows_kernel(T* __restrict__ out, const T* __restrict__ h, 
   for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + r * W + i, ldf(src + i) * sc);
 }
 
+// ---- all-experts form of input-weighted experts: out[e, t] = w[t, j] * h[t] where expert e is
+// row t's j-th choice, zero rows elsewhere. grid (E * T)
+template <typename T>
+__global__ void moe_spread_rows_kernel(T* __restrict__ out, const T* __restrict__ h, const int* __restrict__ idx,
+                                       const float* __restrict__ w, int T_, int W, int top) {
+  const int64_t r = blockIdx.x;
+  const int e = (int)(r / T_), t = (int)(r - (int64_t)e * T_);
+  float sc = 0.f;
+  for (int j = 0; j < top; ++j)
+    if (idx[t * top + j] == e) sc = w[t * top + j];
+  const T* src = h + (int64_t)t * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + r * W + i, sc != 0.f ? ldf(src + i) * sc : 0.f);
+}
+
 template <typename T>
 __global__ void scale_rows_v8_kernel(T* __restrict__ out, const T* __restrict__ h,
                                      const int* __restrict__ src_row, const float* __restrict__ scale, int W) {
@@ -504,6 +518,12 @@ extern "C" void seq_launch_moe_combine(void* out, const void* rows, const void* 
   DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(T_), dim3(row_threads(W)), 0, st, (T*)out,
                                         (const T*)rows, (const T*)h, rowidx, w, (const T*)extra,
                                         (const T*)extra_gate, gate_stride, W, top);)
+}
+
+extern "C" void seq_launch_moe_spread_rows(void* out, const void* h, const int* idx, const float* w, int E,
+                                           int T_, int W, int top, int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(moe_spread_rows_kernel<T>, dim3(E * T_), dim3(row_threads(W)), 0, st,
+                                        (T*)out, (const T*)h, idx, w, T_, W, top);)
 }
 
 extern "C" void seq_launch_scale_rows(void* out, const void* h, const int* src_row, const float* scale, int n,

@@ -707,6 +707,15 @@ def scale_rows(h, src_row, scale) -> torch.Tensor:
     return (h[src_row.long()].float() * scale.float()[:, None]).to(h.dtype)
 
 
+def moe_spread_rows(h, idx, w, experts: int) -> torch.Tensor:
+    """[experts, T, W]: expert e's input rows in the all-experts form of
+    input-weighted experts, w[t, j] * h[t] where e is row t's j-th choice and
+    zero rows elsewhere."""
+    T = h.shape[0]
+    wsel = torch.zeros((T, experts), dtype=torch.float32, device=h.device).scatter_(1, idx.long(), w.float())
+    return (h.float()[None] * wsel.t()[:, :, None]).to(h.dtype)
+
+
 def gelu_tanh(x) -> torch.Tensor:
     """0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) in fp32, in x's dtype."""
     z = x.float()

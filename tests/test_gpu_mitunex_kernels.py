@@ -82,6 +82,16 @@ def test_scale_rows(dtype, W):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_spread_rows_for_the_all_experts_form(dtype):
+    T, W, E, top = 9, 52, 5, 2
+    h = rnd(T, W, dtype=dtype)
+    idx = torch.stack([torch.randperm(E, generator=torch.Generator().manual_seed(i))[:top] for i in range(T)])
+    idx = idx.to(torch.int32).to(DEV)
+    w = torch.rand(T, top, device=DEV) + 0.05
+    close(ops.moe_spread_rows(h, idx, w, E), torch_ref.moe_spread_rows(h, idx, w, E), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("score,renorm,corr", [("sigmoid", False, False), ("sigmoid", True, True),
                                                ("softmax", True, True), ("softmax", False, False)])
 def test_router_variants(dtype, score, renorm, corr):
@@ -167,7 +177,8 @@ def test_latent_attention_kernels(dtype, H, D, R, C, mask):
     c = _latent_case(dtype, H, D, R, C, 16, [33, 1, 2, 1, 70], [0, 52, 15, 0, 45], seed=H + C)
     ref = torch_ref.attn_latent_paged(c["q_abs"], c["q"], c["cache"], c["bt"], c["tseg"], c["pos"], 0.17, mask,
                                       c["gate"], D)
-    for kw in [dict(use_mfma=False), dict(tile_rows=0), dict(tile_rows=1)]:
+    for kw in [dict(use_mfma=False), dict(tile_rows=0), dict(tile_rows=1, key_splits=-1), dict(tile_rows=1),
+               dict(tile_rows=1, key_splits=3), dict(tile_rows=1, key_splits=50)]:
         out = ops.attn_latent_paged(c["q_abs"], c["q"], c["cache"], c["bt"], c["tseg"], c["pos"], 0.17, mask,
                                     c["gate"], D, **kw)
         close(out, ref, dtype)
