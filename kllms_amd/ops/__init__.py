@@ -627,8 +627,9 @@ def attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale
             reach = min(reach, block_tables.shape[1] * cache.shape[2])
             tiles = max(1, (reach + 31) // 32)
             groups = T * ((H + 31) // 32)
-            ns = key_splits or max(1, min((tiles + 1) // 2, 1024 // max(1, groups)))
-            ns = max(1, min(ns, tiles))
+            # about four tiles per workgroup, and no more workgroups than two per compute unit
+            ns = key_splits or max(1, min((tiles + 3) // 4, 512 // max(1, groups)))
+            ns = max(1, min(ns, tiles, 64))
         f = torch.float32
         part_o = torch.empty((T, H, ns, C), dtype=f, device=q.device) if ns > 1 else _none(q, f)
         part_ml = torch.empty((T, H, ns, 2), dtype=f, device=q.device) if ns > 1 else _none(q, f)

@@ -193,7 +193,7 @@ void attn_latent_paged(torch::Tensor out, torch::Tensor q_abs, torch::Tensor q, 
     CHECK_F32C(part_o); CHECK_F32C(part_ml);
     TORCH_CHECK(part_o.dim() == 4 && part_o.size(0) == T && part_o.size(1) == H && part_o.size(3) == C);
     nsplit = (int)part_o.size(2);
-    TORCH_CHECK(nsplit >= 1 && nsplit <= 1024 && part_ml.numel() == (int64_t)T * H * nsplit * 2);
+    TORCH_CHECK(nsplit >= 1 && nsplit <= 64 && part_ml.numel() == (int64_t)T * H * nsplit * 2);
   }
   if (T == 0) return;
   seq_launch_attn_latent_paged(out.data_ptr(), q_abs.data_ptr(), q.data_ptr(), cache.data_ptr(),

@@ -4,7 +4,7 @@
 // dot product with j's cached row, and its output is the weighted sum of the
 // latents (W_uv is applied afterwards). The kernels here:
 //   latent_kv_store    query rotation in place, latent RMS norm, key-part
-//                      rotation, paged store of the cached row
+//                      rotation, paged store of the cached row (one launch)
 //   attn_latent_paged  sliding-window softmax attention over the paged rows
 //     - a plain kernel (any size, bf16 or fp32; the exact-mode path)
 //     - an MFMA kernel (bf16): 32 (row, head) query columns of one workgroup
@@ -15,38 +15,37 @@
 #include "seq_common.h"
 
 // ---- step input ----------------------------------------------------------------
-// grid (T, H + 1), one wave. Blocks 0..H-1: rotate the last R entries of query
-// head h (interleaved pairs, angle = float(pos) * inv_freq[i]) in place. Block
-// H: the token's down-projection row dkv [C + R] -> cache row
+// One workgroup of 256 threads per row. All threads: rotate the last R entries of
+// every query head (interleaved pairs, angle = float(pos) * inv_freq[i]) in
+// place. Then the row's down-projection dkv [C + R] -> cache row
 // [rms(dkv[:C]) * w | rotate(dkv[C:])].
 template <typename T>
-__global__ void latent_kv_store_kernel(T* __restrict__ q, const T* __restrict__ dkv,
-                                       const float* __restrict__ w, float eps,
-                                       const int64_t* __restrict__ positions,
-                                       const float* __restrict__ inv_freq, T* __restrict__ cache,
-                                       const int64_t* __restrict__ slots, int H, int D, int R, int C,
-                                       int q_stride, int dkv_stride) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ void __launch_bounds__(256) latent_kv_store_kernel(
+    T* __restrict__ q, const T* __restrict__ dkv, const float* __restrict__ w, float eps,
+    const int64_t* __restrict__ positions, const float* __restrict__ inv_freq, T* __restrict__ cache,
+    const int64_t* __restrict__ slots, int H, int D, int R, int C, int q_stride, int dkv_stride) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
   const float pos = (float)positions[t];
-  if (h < H) {
-    T* row = q + (int64_t)t * q_stride + (int64_t)h * (D + R) + D;
-    for (int i = lane; i < R / 2; i += WAVE) {
-      float s, c;
-      sincosf(pos * inv_freq[i], &s, &c);
-      const float u = ldf(row + 2 * i), v = ldf(row + 2 * i + 1);
-      stf(row + 2 * i, u * c - v * s);
-      stf(row + 2 * i + 1, v * c + u * s);
-    }
-    return;
-  }
+  const int R2 = R / 2;
   const T* src = dkv + (int64_t)t * dkv_stride;
   T* dst = cache + slots[t] * (int64_t)(C + R);
   float ss = 0.f;
-  for (int i = lane; i < C; i += WAVE) { const float x = ldf(src + i); ss += x * x; }
-  ss = wave_sum(ss);
+  for (int i = tid; i < C; i += blockDim.x) { const float x = ldf(src + i); ss += x * x; }
+  T* qrow = q + (int64_t)t * q_stride + D;
+  for (int idx = tid; idx < H * R2; idx += blockDim.x) {
+    const int h = idx / R2, i = idx - h * R2;
+    T* row = qrow + (int64_t)h * (D + R);
+    float s, c;
+    sincosf(pos * inv_freq[i], &s, &c);
+    const float u = ldf(row + 2 * i), v = ldf(row + 2 * i + 1);
+    stf(row + 2 * i, u * c - v * s);
+    stf(row + 2 * i + 1, v * c + u * s);
+  }
+  ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)C + eps);
-  for (int i = lane; i < C; i += WAVE) stf(dst + i, ldf(src + i) * r * w[i]);
-  for (int i = lane; i < R / 2; i += WAVE) {
+  for (int i = tid; i < C; i += blockDim.x) stf(dst + i, ldf(src + i) * r * w[i]);
+  for (int i = tid; i < R2; i += blockDim.x) {
     float s, c;
     sincosf(pos * inv_freq[i], &s, &c);
     const float u = ldf(src + C + 2 * i), v = ldf(src + C + 2 * i + 1);
@@ -452,9 +451,16 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES, 2) attn_latent_mfma_kernel(
         const int dt = wave + i * LAT_WAVES;
         if (dt < ndt) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int d = dt * 32 + lat_acc_row(r, half);
-            if (d < C) po[d] = o_acc[i][r];
+          for (int g4 = 0; g4 < 4; ++g4) {             // regs 4 g4 .. 4 g4 + 3 hold 4 consecutive dims
+            const int d = dt * 32 + 8 * g4 + 4 * half;
+            if (C % 4 == 0 && d + 4 <= C) {
+              *reinterpret_cast<float4*>(po + d) = make_float4(o_acc[i][4 * g4], o_acc[i][4 * g4 + 1],
+                                                               o_acc[i][4 * g4 + 2], o_acc[i][4 * g4 + 3]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (d + e < C) po[d + e] = o_acc[i][4 * g4 + e];
+            }
           }
         }
       }
@@ -489,27 +495,37 @@ __global__ void __launch_bounds__(WAVE * LAT_WAVES, 2) attn_latent_mfma_kernel(
   }
 }
 
-// Merge of the key shares' partial results: grid (T, H), one wave.
-__global__ void attn_latent_merge_kernel(bfraw* __restrict__ out, const float* __restrict__ part_o,
-                                         const float* __restrict__ part_ml, const bfraw* __restrict__ gate,
-                                         int H, int C, int nsplit, int gate_stride) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+// Merge of the key shares' partial results: grid (T, H), 256 threads. Every
+// thread derives the shares' common maximum; the shares' factors 2^(m_z - M)
+// go through LDS; threads own output dims and sum the shares in a fixed order.
+#define LAT_MAX_SPLIT 64
+__global__ void __launch_bounds__(256) attn_latent_merge_kernel(
+    bfraw* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const bfraw* __restrict__ gate, int H, int C, int nsplit, int gate_stride) {
+  __shared__ float fz[LAT_MAX_SPLIT];
+  __shared__ float lsum;
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int64_t base = ((int64_t)t * H + h) * nsplit;
   float M = -INFINITY;
   for (int z = 0; z < nsplit; ++z) M = fmaxf(M, part_ml[2 * (base + z)]);
-  float Lsum = 0.f;
-  for (int z = 0; z < nsplit; ++z) {
-    const float l = part_ml[2 * (base + z) + 1];
-    if (l > 0.f) Lsum += l * __builtin_amdgcn_exp2f(part_ml[2 * (base + z)] - M);
+  if (tid < nsplit) {
+    const float l = part_ml[2 * (base + tid) + 1];
+    fz[tid] = l > 0.f ? __builtin_amdgcn_exp2f(part_ml[2 * (base + tid)] - M) : 0.f;
   }
-  float gsc = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+  __syncthreads();
+  if (tid == 0) {
+    float L = 0.f;
+    for (int z = 0; z < nsplit; ++z) L += part_ml[2 * (base + z) + 1] * fz[z];
+    lsum = L;
+  }
+  __syncthreads();
+  float gsc = lsum > 0.f ? 1.0f / lsum : 0.f;
   if (gate != nullptr) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
-  for (int d = lane; d < C; d += WAVE) {
+  for (int d = tid; d < C; d += 256) {
+    const float* po = part_o + base * C + d;
     float acc = 0.f;
-    for (int z = 0; z < nsplit; ++z) {
-      const float l = part_ml[2 * (base + z) + 1];
-      if (l > 0.f) acc += part_o[(base + z) * C + d] * __builtin_amdgcn_exp2f(part_ml[2 * (base + z)] - M);
-    }
+#pragma unroll 4
+    for (int z = 0; z < nsplit; ++z) acc += po[(int64_t)z * C] * fz[z];
     stf(out + ((int64_t)t * H + h) * C + d, acc * gsc);
   }
 }
@@ -521,7 +537,7 @@ extern "C" void seq_launch_latent_kv_store(void* q, const void* dkv, const float
                                            const int64_t* positions, const float* inv_freq, void* cache,
                                            const int64_t* slots, int T_, int H, int D, int R, int C,
                                            int q_stride, int dkv_stride, int is_f32, hipStream_t st) {
-  DISPATCH_T(is_f32, hipLaunchKernelGGL(latent_kv_store_kernel<T>, dim3(T_, H + 1), dim3(WAVE), 0, st, (T*)q,
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(latent_kv_store_kernel<T>, dim3(T_), dim3(256), 0, st, (T*)q,
                                         (const T*)dkv, w, eps, positions, inv_freq, (T*)cache, slots, H, D, R, C,
                                         q_stride, dkv_stride);)
 }
@@ -556,7 +572,7 @@ extern "C" void seq_launch_attn_latent_paged(void* out, const void* q_abs, const
                        mask_size, T_, H, D, R, C, BS, bt_stride, qa_stride_t, qa_stride_h, q_stride, gate_stride,
                        tr, hb, vec, qvec, part_o, part_ml);
     if (ns > 1)
-      hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(T_, H), dim3(WAVE), 0, st, (bfraw*)out, part_o, part_ml,
+      hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(T_, H), dim3(256), 0, st, (bfraw*)out, part_o, part_ml,
                          (const bfraw*)gate, H, C, ns, gate_stride);
     return;
   }
