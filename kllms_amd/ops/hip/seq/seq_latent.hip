@@ -143,7 +143,10 @@ __global__ void attn_latent_paged_kernel(T* __restrict__ out, const T* __restric
 // rows x `hb` heads = up to 32 query columns (column c = row c / hb, head
 // h0 + c % hb). Rows of a tile that belong to different sequences are served
 // in turn (one pass over the keys per sequence present in the tile; columns of
-// other sequences are masked out of the pass).
+// other sequences are masked out of the pass). With single-row tiles (steps of
+// decoded tokens) gridDim.z workgroups take contiguous shares of the row's key
+// tiles and leave unnormalised partial results (sums, running max and sum)
+// that attn_latent_merge_kernel combines in a fixed order.
 //
 // Per tile of 32 keys:
 //   all threads stage the 32 cached rows [32][Lp] (zero-padded to a multiple
