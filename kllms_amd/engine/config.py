@@ -46,13 +46,15 @@ class ModelArchConfig(BaseModel):
 
 class RotarySpec(BaseModel):
     """Rotary position parameters of one attention mixer: the first ``dims``
-    dimensions of each head rotate as interleaved pairs (2i, 2i+1) with
-    frequency base^(-2i/dims); ``scaling`` is the banded frequency rescale
+    dimensions of each head rotate in pairs (``layout``) with frequency
+    base^(-2i/dims); ``scaling`` is the banded frequency rescale
     (factor / low / high / original context), None = plain."""
 
     base: float = 10000.0
     dims: int = 0
     scaling: Optional[dict] = None
+    # "pairs": entry 2i rotates with 2i+1; "half": entry i with i + dims/2
+    layout: Literal["pairs", "half"] = "pairs"
 
 
 class BlockAttnSpec(BaseModel):
@@ -153,10 +155,12 @@ class MlstmSpec(BaseModel):
 
 
 class SharedExpertSpec(BaseModel):
-    """A silu-GLU expert that every token passes; its output is scaled by
-    sigmoid of one more projection of the input (a scalar per token)."""
+    """An expert that every token passes; its output is scaled by sigmoid of
+    one more projection of the input (a scalar per token). ``limit`` is the
+    clamp of a clamped-GLU expert (None: as the routed experts' form says)."""
 
     ff: int
+    limit: Optional[float] = None
 
 
 class RoutedExpertsSpec(BaseModel):
@@ -181,6 +185,11 @@ class RoutedExpertsSpec(BaseModel):
     correction: bool = True
     weight_on: Literal["output", "input"] = "output"
     shared: Optional[SharedExpertSpec] = None
+    # the experts' form: silu(gate) * up, or the clamped GLU
+    # min(gate, limit) sigmoid(alpha min(gate, limit)) (clamp(up, +-limit) + 1)
+    act: Literal["silu", "clamped"] = "silu"
+    limit: float = 0.0
+    alpha: float = 1.702
 
 
 class BigramSpec(BaseModel):
@@ -443,6 +452,161 @@ def _mitunex_preset(vocab, width, depth, heads, dim, rot_dim, vdim, kv_rank, mas
                              logit_scale=1.5, logit_softcap=30.0)
 
 
+class PoolWindowAttnSpec(BaseModel):
+    """GQA softmax attention over a sliding window of ``mask_size`` positions
+    (0 = plain causal) plus, when ``pool`` > 0, one key and value per aligned
+    block of ``pool`` positions that lies wholly before the window: the means
+    of the block's cached keys and values. q and k pass an RMS norm over the
+    whole projection (all heads at once, one weight per entry) before the
+    rotation; scores are soft-capped at ``softcap`` (0 = none). ``kv_from``:
+    the layer has no key/value projections and reads the cache of that
+    earlier layer (own queries, mask and pooling)."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0
+    mask_size: int = 0
+    pool: int = 0
+    rot: RotarySpec = Field(default_factory=lambda: RotarySpec(layout="half"))
+    kv_from: Optional[int] = None
+
+
+class Mamba2Spec(BaseModel):
+    """State-space mixer with a scalar decay per head and token:
+    S <- exp(-exp(A_h) dt) S + dt B x^T, y = S^T C + D_h x; x, B, C pass a
+    short causal convolution of ``conv`` taps with bias and silu; B and C are
+    shared by the heads of a group; the output is gated by silu(z) and then
+    RMS-normed in ``norm_groups`` equal parts."""
+
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+
+
+class PironexLayerSpec(BaseModel):
+    type: Literal["attention", "mamba2", "latent_attention"]
+    attention: Optional[PoolWindowAttnSpec] = None
+    mamba2: Optional[Mamba2Spec] = None
+    latent: Optional[LatentAttnSpec] = None
+    mlp: Optional[RoutedExpertsSpec] = None
+
+
+class PironexArchConfig(BaseModel):
+    """A decoder whose sublayers are layer-normed before and after,
+    x <- x + ln(sublayer(canon(ln(x)))), where canon adds a short causal
+    convolution over time to the sublayer's input; after every layer the
+    stream is replaced by a learned weighted sum of the embedding output and
+    all layer results so far. Mixers: windowed attention with pooled blocks
+    (optionally on another layer's cache), mamba2, latent attention;
+    feed-forward: routed clamped-GLU experts with a gated shared expert, or
+    none. The LM head is the embedding table. Every size comes from the
+    checkpoint's config.json."""
+
+    arch: Literal["pironex"] = "pironex"
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    canon_taps: int = 1
+    layers: List[PironexLayerSpec]
+    max_position_embeddings: int = 1 << 24
+    tie_word_embeddings: bool = True
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_checkpoint_config(cls, d: dict, shapes: Optional[dict] = None) -> "PironexArchConfig":
+        """Parse the family's config.json (keys: vocab, width, norm.eps,
+        embedding.scale, canon.taps, layers[].type / .mixer / .mlp)."""
+        layers = []
+        for li, spec in enumerate(d["layers"]):
+            m = spec["mixer"]
+            kind = spec["type"]
+            mlp = spec.get("mlp")
+            ff = None
+            if mlp:
+                if mlp.get("kind", "moe") != "moe":
+                    raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+                r, sh = mlp["router"], mlp.get("shared")
+                ff = RoutedExpertsSpec(experts=r["experts"], top=r["top"], ff=mlp["expert"]["ff"], score="softmax",
+                                       renormalize=True, correction=False, act="clamped",
+                                       limit=mlp["expert"]["limit"],
+                                       shared=SharedExpertSpec(ff=sh["ff"], limit=sh["limit"]) if sh else None)
+            mask = m.get("mask") or {}
+            rot = m.get("rot") or {}
+            if kind == "attention":
+                src = m.get("kv_from")
+                if src is not None:
+                    other = d["layers"][src] if 0 <= src < li else None
+                    if other is None or other["type"] != "attention" or other["mixer"].get("kv_from") is not None:
+                        raise ValueError(f"layer {li}: kv_from {src} does not name an earlier attention layer "
+                                         f"with keys and values of its own")
+                layers.append(PironexLayerSpec(type=kind, mlp=ff, attention=PoolWindowAttnSpec(
+                    heads=m["heads"], kv_heads=m["kv_heads"], dim=m["dim"], vdim=m["vdim"], scale=m["scale"],
+                    softcap=m.get("softcap") or 0.0, mask_size=mask.get("size") or 0, pool=mask.get("pool") or 0,
+                    rot=RotarySpec(base=rot.get("base", 10000.0), dims=rot.get("dims") or 0, layout="half"),
+                    kv_from=src)))
+            elif kind == "mamba2":
+                layers.append(PironexLayerSpec(type=kind, mlp=ff, mamba2=Mamba2Spec(
+                    heads=m["heads"], vdim=m["vdim"], state=m["state"], groups=m["groups"], conv=m["conv"],
+                    norm_groups=m.get("norm_groups") or 1)))
+            elif kind == "latent_attention":
+                att = LatentAttnSpec(heads=m["heads"], dim=m["dim"], rot_dim=m["rot_dim"], vdim=m["vdim"],
+                                     kv_rank=m["kv_rank"], scale=m["scale"], mask_size=mask.get("size") or 0,
+                                     rot=RotarySpec(base=rot.get("base", 10000.0),
+                                                    dims=rot.get("dims") or m["rot_dim"]),
+                                     head_gate=False)
+                if att.rot.dims != att.rot_dim:
+                    raise ValueError("the rotated part of a latent-attention head is rotated whole")
+                layers.append(PironexLayerSpec(type=kind, mlp=ff, latent=att))
+            else:
+                raise ValueError(f"unknown layer type {kind!r}")
+        return cls(vocab_size=d["vocab"], hidden_size=d["width"], norm_eps=d["norm"]["eps"],
+                   embed_scale=(d.get("embedding") or {}).get("scale", 1.0),
+                   canon_taps=(d.get("canon") or {}).get("taps", 1), layers=layers)
+
+
+def _pironex_preset(vocab, width, depth, heads, kv_heads, dim, mask, pool, m_heads, m_vdim, m_state, m_groups,
+                    l_heads, l_dim, l_rot, l_vdim, l_rank, l_mask, experts, top, expert_ff, shared_ff,
+                    pattern="mlamla", taps=3) -> PironexArchConfig:
+    """Random-init presets of the family: ``pattern`` repeats over the depth
+    ('m' mamba2, 'l' latent attention, 'a' attention; a later 'a' reads the
+    first one's keys and values)."""
+    import math as _math
+
+    layers = []
+    first_att = None
+    for i in range(depth):
+        c = pattern[i % len(pattern)]
+        ff = RoutedExpertsSpec(experts=experts, top=top, ff=expert_ff, score="softmax", renormalize=True,
+                               correction=False, act="clamped", limit=7.0,
+                               shared=SharedExpertSpec(ff=shared_ff, limit=7.0) if shared_ff else None)
+        if c == "a":
+            layers.append(PironexLayerSpec(type="attention", mlp=ff, attention=PoolWindowAttnSpec(
+                heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=1.0 / _math.sqrt(dim), softcap=50.0,
+                mask_size=mask, pool=pool, rot=RotarySpec(base=500000.0, dims=dim // 2, layout="half"),
+                kv_from=first_att)))
+            if first_att is None:
+                first_att = i
+        elif c == "m":
+            layers.append(PironexLayerSpec(type="mamba2", mlp=ff, mamba2=Mamba2Spec(
+                heads=m_heads, vdim=m_vdim, state=m_state, groups=m_groups, conv=4, norm_groups=m_groups)))
+        else:
+            layers.append(PironexLayerSpec(type="latent_attention", mlp=ff, latent=LatentAttnSpec(
+                heads=l_heads, dim=l_dim, rot_dim=l_rot, vdim=l_vdim, kv_rank=l_rank,
+                scale=1.0 / _math.sqrt(l_dim + l_rot), mask_size=l_mask,
+                rot=RotarySpec(base=1e6, dims=l_rot), head_gate=False)))
+    return PironexArchConfig(vocab_size=vocab, hidden_size=width, embed_scale=1.0, canon_taps=taps, layers=layers)
+
+
 class HybridLayerSpec(BaseModel):
     type: Literal["parallel", "channel_delta"]
     parallel: Optional[ParallelMixerSpec] = None
@@ -653,6 +817,26 @@ MODEL_PRESETS: dict = {
     "mitunex-1b-l6": _mitunex_preset(
         vocab=32000, width=2048, depth=6, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, mask=1024,
         ff=8192, experts=8, top=2, expert_ff=4096, shared_ff=1024),
+    # Pironex family (layer-normed sublayers with a short input convolution,
+    # depth-weighted stream; mamba2, latent attention and windowed attention
+    # with pooled blocks; routed clamped-GLU experts)
+    "tiny-pironex": _pironex_preset(
+        vocab=512, width=64, depth=6, heads=4, kv_heads=2, dim=16, mask=24, pool=4, m_heads=4, m_vdim=16,
+        m_state=8, m_groups=2, l_heads=4, l_dim=16, l_rot=8, l_vdim=24, l_rank=32, l_mask=24, experts=6, top=2,
+        expert_ff=48, shared_ff=40),
+    "mid-pironex": _pironex_preset(
+        vocab=2048, width=512, depth=3, heads=4, kv_heads=2, dim=128, mask=256, pool=16, m_heads=8, m_vdim=64,
+        m_state=64, m_groups=2, l_heads=8, l_dim=64, l_rot=32, l_vdim=64, l_rank=128, l_mask=256, experts=8,
+        top=2, expert_ff=256, shared_ff=256, pattern="mla"),
+    # layer shapes of real models at reduced depth, beside llama-/mitunex-{1b,8b}-l6
+    "pironex-8b-l6": _pironex_preset(
+        vocab=32000, width=4096, depth=6, heads=32, kv_heads=8, dim=128, mask=2048, pool=64, m_heads=64,
+        m_vdim=64, m_state=128, m_groups=8, l_heads=32, l_dim=128, l_rot=64, l_vdim=128, l_rank=512, l_mask=2048,
+        experts=8, top=2, expert_ff=7168, shared_ff=2048),
+    "pironex-1b-l6": _pironex_preset(
+        vocab=32000, width=2048, depth=6, heads=16, kv_heads=4, dim=128, mask=1024, pool=64, m_heads=32,
+        m_vdim=64, m_state=128, m_groups=4, l_heads=16, l_dim=128, l_rot=64, l_vdim=128, l_rank=512, l_mask=1024,
+        experts=8, top=2, expert_ff=4096, shared_ff=1024),
 }
 
 
@@ -755,11 +939,11 @@ class EngineConfig(BaseModel):
         with open(cfg_path) as f:
             hf = json.load(f)
         family = str(hf.get("architecture", "")).lower()
-        if family in ("zutalix", "medilix", "mitunex"):
+        if family in ("zutalix", "medilix", "mitunex", "pironex"):
             from .weights import safetensors_shapes
 
             reader = {"zutalix": HybridArchConfig, "medilix": MedilixArchConfig,
-                      "mitunex": MitunexArchConfig}[family]
+                      "mitunex": MitunexArchConfig, "pironex": PironexArchConfig}[family]
             return reader.from_checkpoint_config(hf, safetensors_shapes(os.path.dirname(cfg_path)))
         arch = "mixtral" if "mixtral" in hf.get("model_type", "").lower() or hf.get("num_local_experts") else "llama"
         return ModelArchConfig(

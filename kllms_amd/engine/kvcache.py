@@ -213,20 +213,32 @@ class LayerCacheSpec:
     recurrent state matrix per head; conv = (channels, history) of carried
     convolution inputs; shift = width of the previous token's layer input
     (token-shift mixers); tok = the previous token id (hashed n-gram
-    embeddings). None / False = the layer has no such state."""
+    embeddings). kv_of = index of the cache entry whose paged keys and values
+    this layer reads instead of keeping its own. pool = (kv_heads, key_dim,
+    value_dim, block) of pooled keys and values: the fp32 mean over every
+    aligned run of ``block`` positions, kept page by page beside the tokens
+    (an entry lives in the page of its run's last token). canon = (count,
+    width, history): fp32 inputs of ``count`` short convolutions over the
+    layer's normed stream. None / False = the layer has no such state."""
 
     kv: Optional[Tuple[int, int, int]] = None
     rec: Optional[Tuple[int, int, int]] = None
     conv: Optional[Tuple[int, int]] = None
     shift: Optional[int] = None
     tok: bool = False
+    kv_of: Optional[int] = None
+    pool: Optional[Tuple[int, int, int, int]] = None
+    canon: Optional[Tuple[int, int, int]] = None
 
 
 @dataclass
 class LayerState:
     """One layer's device tensors: paged k/v [NB, G, BS, D|Dv], recurrent
     state [slots, H, D, V] fp32, convolution history [slots, K-1, C], previous
-    layer input [slots, W], previous token id [slots] int32."""
+    layer input [slots, W], previous token id [slots] int32, pooled keys /
+    values [NB, G, ceil(BS / block), D|Dv] fp32, normed-stream history
+    [slots, count, K-1, W] fp32. ``shared_kv``: k and v belong to another
+    entry."""
 
     k: Optional[torch.Tensor] = None
     v: Optional[torch.Tensor] = None
@@ -234,10 +246,19 @@ class LayerState:
     conv: Optional[torch.Tensor] = None
     shift: Optional[torch.Tensor] = None
     tok: Optional[torch.Tensor] = None
+    pool_k: Optional[torch.Tensor] = None
+    pool_v: Optional[torch.Tensor] = None
+    canon: Optional[torch.Tensor] = None
+    shared_kv: bool = False
 
     def slot_tensors(self):
         """The per-slot tensors (first dim = slot), for copying a slot."""
-        return [t for t in (self.rec, self.conv, self.shift, self.tok) if t is not None]
+        return [t for t in (self.rec, self.conv, self.shift, self.tok, self.canon) if t is not None]
+
+    def block_tensors(self):
+        """The per-page tensors this entry owns (first dim = page), for copying a page."""
+        own = [] if self.shared_kv else [self.k, self.v]
+        return [t for t in own + [self.pool_k, self.pool_v] if t is not None]
 
 
 class StateSlotPool:
@@ -301,13 +322,30 @@ class HybridStateCache(PagedKVCache):
                 st.shift = torch.zeros(num_slots, sp.shift, device=device, dtype=dtype)
             if sp.tok:
                 st.tok = torch.zeros(num_slots, device=device, dtype=torch.int32)
+            if sp.kv_of is not None:
+                src = self.layers[sp.kv_of]
+                assert sp.kv is None and src.k is not None and not src.shared_kv
+                st.k, st.v, st.shared_kv = src.k, src.v, True
+            if sp.pool is not None:
+                g, d, dv, run = sp.pool
+                per_page = (block_size + run - 1) // run
+                st.pool_k = torch.zeros(num_blocks, g, per_page, d, device=device, dtype=torch.float32)
+                st.pool_v = torch.zeros(num_blocks, g, per_page, dv, device=device, dtype=torch.float32)
+            if sp.canon is not None:
+                n, w, hist = sp.canon
+                st.canon = torch.zeros(num_slots, n, hist, w, device=device, dtype=torch.float32)
             self.layers.append(st)
         self.allocator = BlockAllocator(num_blocks)
         self.slots = StateSlotPool(num_slots)
 
     @staticmethod
     def bytes_per_block(specs: List[LayerCacheSpec], block_size: int, elem: int) -> int:
-        return sum(sp.kv[0] * block_size * (sp.kv[1] + sp.kv[2]) * elem for sp in specs if sp.kv)
+        n = sum(sp.kv[0] * block_size * (sp.kv[1] + sp.kv[2]) * elem for sp in specs if sp.kv)
+        for sp in specs:
+            if sp.pool:
+                g, d, dv, run = sp.pool
+                n += g * ((block_size + run - 1) // run) * (d + dv) * 4
+        return n
 
     @staticmethod
     def bytes_per_slot(specs: List[LayerCacheSpec], elem: int) -> int:
@@ -321,6 +359,8 @@ class HybridStateCache(PagedKVCache):
                 n += sp.shift * elem
             if sp.tok:
                 n += 4
+            if sp.canon:
+                n += sp.canon[0] * sp.canon[1] * sp.canon[2] * 4
         return n
 
     def layer_caches(self) -> List[LayerState]:
@@ -329,9 +369,8 @@ class HybridStateCache(PagedKVCache):
     def _copy_block(self, src: int) -> int:
         dst = self.allocator.alloc()
         for st in self.layers:
-            if st.k is not None:
-                st.k[dst].copy_(st.k[src])
-                st.v[dst].copy_(st.v[src])
+            for t in st.block_tensors():
+                t[dst].copy_(t[src])
         return dst
 
     def open_sequence(self) -> SequenceKV:

@@ -38,9 +38,15 @@ class ListedLayerLM(nn.Module):
             dst = m.get(name)
             if dst is None:
                 raise RuntimeError(f"checkpoint tensor {name!r} has no place in this model")
-            if tuple(dst.shape) != tuple(t.shape):
-                raise RuntimeError(f"{name}: checkpoint shape {tuple(t.shape)} != model {tuple(dst.shape)}")
-            dst.copy_(t.to(dst.dtype))
+            # a list: the checkpoint tensor's rows are dealt to several parameter slices in turn
+            parts = dst if isinstance(dst, (list, tuple)) else [dst]
+            shape = (sum(d.shape[0] for d in parts),) + tuple(parts[0].shape[1:])
+            if shape != tuple(t.shape) or any(tuple(d.shape[1:]) != shape[1:] for d in parts):
+                raise RuntimeError(f"{name}: checkpoint shape {tuple(t.shape)} != model {shape}")
+            r = 0
+            for d in parts:
+                d.copy_(t[r:r + d.shape[0]].to(d.dtype))
+                r += d.shape[0]
             seen.add(name)
         missing = sorted(set(m) - seen)
         if missing:

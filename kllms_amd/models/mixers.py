@@ -25,8 +25,8 @@ import torch.nn.functional as F
 
 from .. import ops
 from ..engine.config import (ActFFSpec, BlockAttnSpec, ChannelDeltaSpec, DecayLinearAttnSpec, GluSpec,
-                             LatentAttnSpec, MaskedAttnSpec, MlstmSpec, ParallelMixerSpec, RotarySpec,
-                             RoutedExpertsSpec, WkvSpec)
+                             LatentAttnSpec, Mamba2Spec, MaskedAttnSpec, MlstmSpec, ParallelMixerSpec,
+                             PoolWindowAttnSpec, RotarySpec, RoutedExpertsSpec, WkvSpec)
 from ..engine.kvcache import LayerCacheSpec, LayerState
 
 
@@ -447,6 +447,122 @@ class LatentAttention(nn.Module):
         return m
 
 
+class PoolWindowAttention(nn.Module):
+    """GQA softmax attention over the paged cache: a sliding window of
+    ``mask_size`` tokens and, before it, one pooled key / value per aligned
+    run of ``pool`` tokens that the window has left behind entirely (the fp32
+    means of the run's cached keys and values, kept in a pooled cache that is
+    filled whenever a step completes a run). q and k are RMS-normed over the
+    whole projection, then rotated (entry i with i + dims/2); scores are
+    soft-capped. A layer with ``kv_from`` projects queries only and reads the
+    keys and values another layer cached in this step; its pooled cache is
+    its own (its run length may differ)."""
+
+    def __init__(self, spec: PoolWindowAttnSpec, hidden: int, eps: float, dtype):
+        super().__init__()
+        assert spec.heads % spec.kv_heads == 0 and spec.rot.dims % 2 == 0 and spec.rot.dims <= spec.dim
+        assert spec.rot.layout == "half" and not spec.rot.scaling
+        self.spec = spec
+        self.eps = eps
+        self.own_kv = spec.kv_from is None
+        parts = [("q", spec.heads * spec.dim)]
+        if self.own_kv:
+            parts += [("k", spec.kv_heads * spec.dim), ("v", spec.kv_heads * spec.vdim)]
+        self.inp = FusedInput(hidden, parts, dtype)
+        self.q_norm = _param(spec.heads * spec.dim, dtype=torch.float32)
+        self.k_norm = _param(spec.kv_heads * spec.dim, dtype=torch.float32) if self.own_kv else None
+        self.o_proj = _param(hidden, spec.heads * spec.vdim, dtype=dtype)
+        self.register_buffer("inv_freq", rotary_inv_freq(spec.rot), persistent=False)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        kv = (sp.kv_heads, sp.dim, sp.vdim)
+        return LayerCacheSpec(kv=kv if self.own_kv else None, kv_of=sp.kv_from,
+                              pool=kv + (sp.pool,) if sp.pool > 0 and sp.mask_size > 0 else None)
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        T = h.shape[0]
+        y = self.inp(h)
+        s = self.inp.split
+        q = s(y, "q").unflatten(1, (sp.heads, sp.dim))
+        k = v = None
+        if self.own_kv:
+            k = s(y, "k").unflatten(1, (sp.kv_heads, sp.dim))
+            v = s(y, "v").unflatten(1, (sp.kv_heads, sp.vdim))
+        ops.qk_fullnorm_rope_store(q, k, v, self.q_norm, self.k_norm, self.eps, batch.positions, self.inv_freq,
+                                   st.k, st.v, batch.slot_mapping)
+        run = sp.pool if st.pool_k is not None else 0
+        if run:
+            ops.pool_kv_update(st.k, st.v, st.pool_k, st.pool_v, batch.block_tables, batch.token_seg,
+                               batch.positions, run)
+        att = ops.attn_window_pool_paged(q, st.k, st.v, st.pool_k, st.pool_v, batch.block_tables, batch.token_seg,
+                                         batch.positions, sp.scale, sp.softcap, sp.mask_size, run)
+        return F.linear(att.reshape(T, -1), self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + n: self.inp.slot(n) for n in self.inp.parts}
+        m[pre + "q.norm"] = self.q_norm
+        if self.own_kv:
+            m[pre + "k.norm"] = self.k_norm
+        m[pre + "o"] = self.o_proj
+        return m
+
+
+class Mamba2Mixer(nn.Module):
+    """State-space mixer. One input GEMM gives [z | x | B | C | dt]; x, B, C
+    pass a short causal convolution (with bias) and silu together; per head h
+    of group g, with d = softplus(dt + dt_bias) in fp32:
+        S <- exp(-exp(A_h) d) S + d B_g x_h^T,   y_h = S^T C_g + D_h x_h
+    then y * silu(z), RMS norm in ``norm_groups`` equal parts, norm weight,
+    projection. State: S [H, N, P] fp32 and the convolution's last inputs."""
+
+    def __init__(self, spec: Mamba2Spec, hidden: int, eps: float, dtype):
+        super().__init__()
+        assert spec.heads % spec.groups == 0 and (spec.heads * spec.vdim) % spec.norm_groups == 0
+        self.spec = spec
+        self.eps = eps
+        self.inner = spec.heads * spec.vdim
+        self.gn = spec.groups * spec.state
+        self.ch = self.inner + 2 * self.gn
+        self.inp = FusedInput(hidden, [("z", self.inner), ("xbc", self.ch), ("dt", spec.heads)], dtype)
+        self.conv = nn.Parameter(torch.zeros(spec.conv, self.ch, dtype=torch.float32), requires_grad=False)
+        self.conv_bias = _param(self.ch, dtype=torch.float32)
+        self.dt_bias = _param(spec.heads, dtype=torch.float32)
+        self.A_log = _param(spec.heads, dtype=torch.float32)
+        self.D = _param(spec.heads, dtype=torch.float32)
+        self.norm = _param(self.inner, dtype=torch.float32)
+        self.o_proj = _param(hidden, self.inner, dtype=dtype)
+
+    def cache_spec(self) -> LayerCacheSpec:
+        sp = self.spec
+        return LayerCacheSpec(rec=(sp.heads, sp.state, sp.vdim), conv=(self.ch, sp.conv - 1))
+
+    def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
+        sp = self.spec
+        y = self.inp(h)
+        s = self.inp.split
+        xbc = ops.causal_conv_silu(s(y, "xbc"), self.conv, st.conv, batch.state_slots, batch.cu_seqlens,
+                                   batch.seg_start, batch.token_seg, self.conv_bias)
+        o = ops.ssd_recurrence(xbc[:, :self.inner].unflatten(1, (sp.heads, sp.vdim)),
+                               xbc[:, self.inner:self.inner + self.gn].unflatten(1, (sp.groups, sp.state)),
+                               xbc[:, self.inner + self.gn:].unflatten(1, (sp.groups, sp.state)),
+                               s(y, "dt"), self.dt_bias, self.A_log, self.D, st.rec, batch.state_slots,
+                               batch.cu_seqlens, batch.seg_start)
+        r = ops.gate_group_rmsnorm(o.view(o.shape[0], sp.norm_groups, -1), self.norm, s(y, "z"), self.eps,
+                                   self.o_proj.dtype)
+        return F.linear(r, self.o_proj)
+
+    def checkpoint_map(self, pre: str) -> Dict[str, torch.Tensor]:
+        m = {pre + "in": [self.inp.slot("z"), self.inp.slot("xbc"), self.inp.slot("dt")]}
+        m[pre + "conv"] = self.conv.t()
+        m[pre + "conv.b"] = self.conv_bias
+        for n in ("dt_bias", "A_log", "D", "norm"):
+            m[pre + n] = getattr(self, n)
+        m[pre + "o"] = self.o_proj
+        return m
+
+
 class ActFF(nn.Module):
     """y = W_down act(W_up h) with the tanh-form gelu."""
 
@@ -571,7 +687,8 @@ class MlstmMixer(nn.Module):
 
 
 class RoutedExperts(nn.Module):
-    """Mixture of silu-GLU experts. The router runs in fp32: scores are the
+    """Mixture of GLU experts (silu(gate) * up, or the clamped form with
+    limits of their own for the routed and the shared expert). The router runs in fp32: scores are the
     softmax over all outputs or the sigmoid of each; the choice is made on
     score (+ correction) within the best groups of neighbouring experts; the
     chosen scores, renormalised or as they are, weigh the experts — their
@@ -613,6 +730,12 @@ class RoutedExperts(nn.Module):
             self.shared_inp = FusedInput(hidden, [("gate", sff), ("up", sff), ("sg", 1)], dtype)
             self.shared_down = _param(hidden, sff, dtype=dtype)
 
+    def _act(self, gate: torch.Tensor, up: torch.Tensor, limit: Optional[float] = None) -> torch.Tensor:
+        sp = self.spec
+        if sp.act == "clamped":
+            return ops.gated_act(gate, up, sp.limit if limit is None else limit, sp.alpha, 1.0)
+        return ops.silu_glu(gate, up)
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         sp = self.spec
         T, W = h.shape
@@ -628,7 +751,7 @@ class RoutedExperts(nn.Module):
             else:
                 xin = h.unsqueeze(0).expand(E, T, W)
             gu = torch.bmm(xin, self.w_gate_up.transpose(1, 2)).view(E * T, 2 * sp.ff)
-            act = ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]).view(E, T, sp.ff)
+            act = self._act(gu[:, :sp.ff], gu[:, sp.ff:]).view(E, T, sp.ff)
             rows = torch.bmm(act, self.w_down.transpose(1, 2)).view(E * T, W)
         else:
             flat = idx.reshape(-1).long().clamp(max=E)                # identity experts sort last
@@ -644,7 +767,7 @@ class RoutedExperts(nn.Module):
             for e, c in enumerate(counts):
                 if c:
                     gu = F.linear(xs[s0:s0 + c], self.w_gate_up[e])
-                    rows[s0:s0 + c] = F.linear(ops.silu_glu(gu[:, :sp.ff], gu[:, sp.ff:]), self.w_down[e])
+                    rows[s0:s0 + c] = F.linear(self._act(gu[:, :sp.ff], gu[:, sp.ff:]), self.w_down[e])
                     s0 += c
             pos = torch.empty(T * top, dtype=torch.int32, device=h.device)
             pos[order] = torch.arange(T * top, dtype=torch.int32, device=h.device)
@@ -653,7 +776,7 @@ class RoutedExperts(nn.Module):
         if self.shared_inp is not None:
             ys = self.shared_inp(h)
             ss = self.shared_inp.split
-            extra = F.linear(ops.silu_glu(ss(ys, "gate"), ss(ys, "up")), self.shared_down)
+            extra = F.linear(self._act(ss(ys, "gate"), ss(ys, "up"), sp.shared.limit), self.shared_down)
             gate = ss(ys, "sg")[:, 0]
         return ops.moe_combine(rows, h, rowidx, None if on_input else w, h.dtype, extra, gate)
 

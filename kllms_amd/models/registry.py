@@ -26,7 +26,11 @@ def model_class(arch: str):
         from .mitunex import MitunexForCausalLM
 
         return MitunexForCausalLM
+    if arch == "pironex":
+        from .pironex import PironexForCausalLM
+
+        return PironexForCausalLM
     raise ValueError(f"no model registered for architecture {arch!r}")
 
 
-ARCHITECTURES = ("llama", "mixtral", "zutalix", "medilix", "mitunex")
+ARCHITECTURES = ("llama", "mixtral", "zutalix", "medilix", "mitunex", "pironex")

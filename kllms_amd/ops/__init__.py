@@ -304,7 +304,8 @@ def attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, s
         _seq().attn_masked_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions,
                                  gate if gate is not None else _none(q), scale, int(mask_kind), int(mask_size),
                                  int(keep_first), bool(sink),
-                                 row_map if row_map is not None else _none(q, torch.int32))
+                                 row_map if row_map is not None else _none(q, torch.int32),
+                                 _none(q, torch.float32), _none(q, torch.float32), 0, 0.0)
         return out
     assert row_map is None and out is None
     return torch_ref.attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale,
@@ -369,12 +370,13 @@ def gated_rmsnorm(o, weight, gate, eps, out_dtype):
     return torch_ref.gated_rmsnorm(o, weight, gate, eps, out_dtype)
 
 
-def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start, token_seg):
+def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start, token_seg, bias=None):
     if _gpu(x):
         y = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-        _seq().causal_conv_silu(y, x, w, conv_state, state_slots, cu_seqlens, seg_start, token_seg)
+        _seq().causal_conv_silu(y, x, w, conv_state, state_slots, cu_seqlens, seg_start, token_seg,
+                                bias if bias is not None else _none(x, torch.float32))
         return y
-    return torch_ref.causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start)
+    return torch_ref.causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start, bias)
 
 
 def gated_delta_rule(q, k, v, beta_logit, a, dt_bias, a_log, state, state_slots, cu_seqlens, seg_start):
@@ -408,16 +410,20 @@ def silu_glu(gate, up):
 
 
 def embed_bigram(ids, table, bigram, scale, mul_prev, mul_cur, buckets, tok_state, state_slots, cu_seqlens,
-                 seg_start, token_seg):
+                 seg_start, token_seg, out=None):
+    """fp32 rows table[id] * scale (+ the hashed bigram row); ``out``: an
+    existing contiguous [T, W] fp32 tensor to fill."""
     if _gpu(table):
-        out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
+        if out is None:
+            out = torch.empty((ids.numel(), table.shape[1]), dtype=torch.float32, device=table.device)
         has = bigram is not None
         _seq().embed_bigram(out, ids, table, bigram if has else _none(table), float(scale), int(mul_prev),
                             int(mul_cur), int(buckets), tok_state if has else _none(table, torch.int32),
                             state_slots, cu_seqlens, seg_start, token_seg)
         return out
-    return torch_ref.embed_bigram(ids, table, bigram, scale, mul_prev, mul_cur, buckets, tok_state,
-                                  state_slots, cu_seqlens, seg_start)
+    x = torch_ref.embed_bigram(ids, table, bigram, scale, mul_prev, mul_cur, buckets, tok_state,
+                               state_slots, cu_seqlens, seg_start)
+    return x if out is None else out.copy_(x)
 
 
 def group_norm_pair(x, a, b, w1, w2, groups, eps, out_dtype):
@@ -647,3 +653,96 @@ def attn_window_sink(q, st, batch, spec, gate):
     mixes alike)."""
     return attn_masked_paged(q, st.k, st.v, batch.block_tables, batch.token_seg, batch.positions, spec.scale,
                              1, spec.mask_size, spec.keep_first, spec.sink, gate)
+
+
+def ln_residual_mix(x_in, a, w_post, eps, x_out, streams=None, n_prev=0, dwa=None):
+    """x_out = x_in + layernorm(a) * w_post (a None: x_in itself); with
+    ``streams`` [L, T, W] the sum is kept as streams[n_prev] and x_out becomes
+    sum_{j <= n_prev} dwa[j] * streams[j]. Returns the (mean, rstd) of every
+    row of x_out, [T, 2] fp32 — what the next layer norm of the stream needs."""
+    if _gpu(x_in):
+        stats = torch.empty((x_in.shape[0], 2), dtype=torch.float32, device=x_in.device)
+        f = _none(x_in, torch.float32)
+        has = streams is not None
+        _seq().ln_residual_mix(x_out, x_in, a if a is not None else f, w_post if a is not None else f, stats,
+                               streams if has else f, dwa if has else f, int(n_prev), eps)
+        return stats
+    return torch_ref.ln_residual_mix(x_in, a, w_post, eps, x_out, streams, n_prev, dwa)
+
+
+def ln_canon(x, stats, w_norm, canon_w, hist, state_slots, cu_seqlens, seg_start, token_seg, out_dtype):
+    """Layer norm of the fp32 stream from its row statistics, times w_norm,
+    plus the short causal convolution of that normed row with its
+    predecessors (canon_w [K, W] taps-major; None = norm only); the
+    sequence's last K-1 normed rows are carried in hist [slots, K-1, W] fp32."""
+    if _gpu(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        f = _none(x, torch.float32)
+        has = canon_w is not None
+        i = _none(x, torch.int32)
+        _seq().ln_canon(out, x, stats, w_norm, canon_w if has else f, hist if has else f,
+                        state_slots if has else i, cu_seqlens if has else i, seg_start if has else i,
+                        token_seg if has else i)
+        return out
+    return torch_ref.ln_canon(x, stats, w_norm, canon_w, hist, state_slots, cu_seqlens, seg_start, out_dtype)
+
+
+def qk_fullnorm_rope_store(q, k, v, wq, wk, eps, positions, inv_freq, k_cache, v_cache, slot_mapping) -> None:
+    """Whole-projection RMS norm of q (in place) and k, half-split rotation of
+    the first 2 * len(inv_freq) entries of every head, normed rotated k and v
+    into the paged caches. k None: q only."""
+    if _gpu(q):
+        e = _none(q)
+        has = k is not None
+        _seq().qk_fullnorm_rope_store(q, k if has else e, v if has else e, wq,
+                                      wk if has else _none(q, torch.float32), eps, positions, inv_freq,
+                                      k_cache if has else e, v_cache if has else e,
+                                      slot_mapping if has else _none(q, torch.long))
+        return
+    torch_ref.qk_fullnorm_rope_store(q, k, v, wq, wk, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
+
+
+def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run: int) -> None:
+    """Means of the cached keys / values of every aligned run of ``run``
+    positions that one of this step's rows completes, into the fp32 pooled
+    caches."""
+    if _gpu(k_cache):
+        _seq().pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, int(run))
+        return
+    torch_ref.pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run)
+
+
+def attn_window_pool_paged(q, k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, scale,
+                           softcap, mask_size, run):
+    """Sliding-window attention over the paged cache with the pooled entries
+    of the runs that lie wholly before the window, soft-capped scores; prompt
+    portions, decoded tokens and mixes alike."""
+    if _gpu(q):
+        out = torch.empty((q.shape[0], q.shape[1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
+        f = _none(q, torch.float32)
+        has = run > 0
+        _seq().attn_masked_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions, _none(q),
+                                 scale, 2, int(mask_size), 0, False, _none(q, torch.int32),
+                                 pool_k if has else f, pool_v if has else f, int(run), float(softcap))
+        return out
+    return torch_ref.attn_window_pool_paged(q, k_cache, v_cache, pool_k, pool_v, block_tables, token_seg,
+                                            positions, scale, softcap, mask_size, run)
+
+
+def ssd_recurrence(x, B, C, dt, dt_bias, a_log, skip, state, state_slots, cu_seqlens, seg_start):
+    """S <- exp(-exp(a_log) d) S + d B x^T, o = S^T C + skip x with
+    d = softplus(dt + dt_bias) per head and token; o [T, H, V] fp32."""
+    if _gpu(x):
+        o = torch.empty((x.shape[0], x.shape[1], x.shape[2]), dtype=torch.float32, device=x.device)
+        _seq().ssd_recurrence(o, x, B, C, dt, dt_bias, a_log, skip, state, state_slots, cu_seqlens, seg_start)
+        return o
+    return torch_ref.ssd_recurrence(x, B, C, dt, dt_bias, a_log, skip, state, state_slots, cu_seqlens, seg_start)
+
+
+def gate_group_rmsnorm(o, weight, gate, eps, out_dtype):
+    """(o * silu(gate)) RMS-normed in groups, times weight: o [T, groups, S] fp32."""
+    if _gpu(o):
+        out = torch.empty((o.shape[0], o.shape[1] * o.shape[2]), dtype=out_dtype, device=o.device)
+        _seq().head_rmsnorm_gate(out, o, weight, gate, eps, 2, _none(o, torch.float32))
+        return out
+    return torch_ref.gate_group_rmsnorm(o, weight, gate, eps, out_dtype)

@@ -390,10 +390,10 @@ def gated_rmsnorm(o, weight, gate, eps, out_dtype) -> torch.Tensor:
     return (y.reshape(T, Gn * S) * torch.sigmoid(gate.float())).to(out_dtype)
 
 
-def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start) -> torch.Tensor:
-    """Per-channel causal convolution over time + silu. x [T,C]; w [K,C]
-    taps-major (last row = current token); conv_state [slots, K-1, C] holds
-    each sequence's last K-1 inputs (oldest first) and is updated."""
+def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start, bias=None) -> torch.Tensor:
+    """Per-channel causal convolution over time (+ bias [C]) + silu. x [T,C];
+    w [K,C] taps-major (last row = current token); conv_state [slots, K-1, C]
+    holds each sequence's last K-1 inputs (oldest first) and is updated."""
     T, C = x.shape
     K = w.shape[0]
     y = torch.empty(T, C, dtype=x.dtype, device=x.device)
@@ -404,10 +404,13 @@ def causal_conv_silu(x, w, conv_state, state_slots, cu_seqlens, seg_start) -> to
         hist = conv_state[sl[b]].float() if st[b] > 0 else torch.zeros(K - 1, C, device=x.device)
         ext = torch.cat([hist, x[s:e].float()], 0)           # [K-1+L, C]
         acc = torch.zeros(e - s, C, device=x.device)
+        if bias is not None:
+            acc += bias.float()
         for j in range(K):
             acc += ext[j:j + (e - s)] * wf[j]
         y[s:e] = torch.nn.functional.silu(acc).to(x.dtype)
-        conv_state[sl[b]] = ext[ext.shape[0] - (K - 1):].to(conv_state.dtype)
+        if K > 1:
+            conv_state[sl[b]] = ext[ext.shape[0] - (K - 1):].to(conv_state.dtype)
     return y
 
 
@@ -786,3 +789,190 @@ def attn_latent_paged(q_abs, q, cache, block_tables, token_seg, positions, scale
             o = o * torch.sigmoid(gate[t].float())[:, None]
         out[t] = o.to(out.dtype)
     return out
+
+
+# --- layer-normed sublayers with an input convolution and a depth-weighted
+# stream; whole-projection q/k norm with half-split rotation; pooled blocks
+# before a sliding window; the mamba2 recurrence -----------------------------------
+
+def _ln_stats(y: torch.Tensor, eps: float) -> torch.Tensor:
+    mu = y.mean(-1)
+    var = (y - mu[:, None]).pow(2).mean(-1)
+    return torch.stack([mu, torch.rsqrt(var + eps)], -1)
+
+
+def ln_residual_mix(x_in, a, w_post, eps, x_out, streams=None, n_prev=0, dwa=None) -> torch.Tensor:
+    """y = x_in + layernorm(a) * w_post (y = x_in when a is None; layernorm
+    subtracts the mean and divides by sqrt(variance + eps), fp32). With
+    ``streams`` [L, T, W]: y is kept as streams[n_prev] and replaced by
+    sum_{j <= n_prev} dwa[j] * streams[j] (summed in that order). y goes to
+    x_out (fp32, may be x_in); returns its per-row (mean, 1/sqrt(var + eps))
+    as [T, 2] fp32, for the norm that reads the stream next."""
+    y = x_in.float()
+    if a is not None:
+        af = a.float()
+        st = _ln_stats(af, eps)
+        y = y + (af - st[:, :1]) * st[:, 1:] * w_post.float()
+    if streams is not None:
+        streams[n_prev].copy_(y)
+        y = torch.zeros_like(y)
+        for j in range(n_prev + 1):
+            y = y + dwa[j].float() * streams[j]
+    x_out.copy_(y)
+    return _ln_stats(y, eps)
+
+
+def ln_canon(x, stats, w_norm, canon_w, hist, state_slots, cu_seqlens, seg_start, out_dtype) -> torch.Tensor:
+    """h = (x - mean) * rstd * w_norm per row (stats [T, 2] from
+    ln_residual_mix); returns h_t + sum_j canon_w[j] * h_{t-K+1+j} in
+    out_dtype (canon_w [K, W] taps-major, last row = the current token; None:
+    h itself). Rows before a segment come from hist [slots, K-1, W] fp32
+    (oldest first; zeros for a fresh sequence), which then takes the
+    sequence's last K-1 rows of h."""
+    h = (x.float() - stats[:, :1]) * stats[:, 1:] * w_norm.float()
+    if canon_w is None:
+        return h.to(out_dtype)
+    K = canon_w.shape[0]
+    out = torch.empty_like(h)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    wf = canon_w.float()
+    for b in range(len(sl)):
+        s, e = cu[b], cu[b + 1]
+        if e == s:
+            continue
+        old = hist[sl[b]].float() if st[b] > 0 else torch.zeros(K - 1, h.shape[1], device=h.device)
+        ext = torch.cat([old, h[s:e]], 0)
+        acc = h[s:e].clone()
+        for j in range(K):
+            acc += ext[j:j + (e - s)] * wf[j]
+        out[s:e] = acc
+        if K > 1:
+            hist[sl[b]] = ext[ext.shape[0] - (K - 1):]
+    return out.to(out_dtype)
+
+
+def qk_fullnorm_rope_store(q, k, v, wq, wk, eps, positions, inv_freq, k_cache, v_cache, slot_mapping) -> None:
+    """RMS norm over the whole projection of q [T, H, D] (weight wq [H*D]; in
+    place) and k [T, G, D] (wk [G*D]), then rotation of the first
+    2*len(inv_freq) entries of every head with entry i paired with
+    i + len(inv_freq) (angle = position * inv_freq[i], fp32). The normed,
+    rotated k and v go to the paged caches. k None: only q (a layer that
+    reads another layer's cache)."""
+    T = q.shape[0]
+    R = inv_freq.numel()
+    ang = positions.to(torch.float32)[:, None] * inv_freq.float()[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+    def norm_rot(t, w):
+        n, d = t.shape[1], t.shape[2]
+        tf = t.float().reshape(T, n * d)
+        tf = tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        tf = tf.view(T, n, d)
+        if R:
+            out = tf.clone()
+            u, x2 = tf[..., :R], tf[..., R:2 * R]
+            out[..., :R] = u * cos - x2 * sin
+            out[..., R:2 * R] = x2 * cos + u * sin
+            tf = out
+        return tf
+
+    if k is not None:
+        BS = k_cache.shape[2]
+        blk, off = slot_mapping // BS, slot_mapping % BS
+        k_cache[blk, :, off, :] = norm_rot(k, wk).to(k_cache.dtype)
+        v_cache[blk, :, off, :] = v.to(v_cache.dtype)
+    q.copy_(norm_rot(q, wq).to(q.dtype))
+
+
+def pool_entry(b: int, run: int, BS: int):
+    """(page index within the sequence, offset within the page's pooled
+    entries) of pooled run b: the page of the run's last token, counted from
+    the first run that ends in that page."""
+    pg = ((b + 1) * run - 1) // BS
+    return pg, b - (pg * BS) // run
+
+
+def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run: int) -> None:
+    """For every row whose position ends an aligned run of ``run`` positions:
+    the fp32 means of the run's cached keys and values go to pool_k / pool_v
+    [NB, G, ceil(BS / run), D|Dv]."""
+    BS = k_cache.shape[2]
+    pos, seg = positions.tolist(), token_seg.tolist()
+    for t, p in enumerate(pos):
+        if (p + 1) % run:
+            continue
+        b = p // run
+        bt = block_tables[seg[t]].long()
+        idx = torch.arange(b * run, (b + 1) * run, device=k_cache.device)
+        pg, off = pool_entry(b, run, BS)
+        pool_k[bt[pg], :, off, :] = k_cache[bt[idx // BS], :, idx % BS, :].float().mean(0)
+        pool_v[bt[pg], :, off, :] = v_cache[bt[idx // BS], :, idx % BS, :].float().mean(0)
+
+
+def attn_window_pool_paged(q, k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, scale,
+                           softcap, mask_size, run, out_dtype=None) -> torch.Tensor:
+    """Softmax attention of packed query rows against the paged cache. Row t
+    at position p sees keys j of its own sequence with 0 <= p - j < mask_size
+    (0 = all j <= p) and, when run > 0, the pooled entry of every aligned run
+    of ``run`` positions that ends at or before p - mask_size. Scores are
+    q . k * scale, soft-capped as cap * tanh(s / cap) when softcap > 0; one
+    softmax over entries and tokens."""
+    T, H, D = q.shape
+    _, G, BS, Dv = v_cache.shape
+    rep = H // G
+    out = torch.empty(T, H, Dv, dtype=out_dtype or q.dtype, device=q.device)
+    pos, seg = positions.tolist(), token_seg.tolist()
+    for t in range(T):
+        p = pos[t]
+        lo = max(0, p - mask_size + 1) if mask_size > 0 else 0
+        idx = torch.arange(lo, p + 1, device=q.device)
+        bt = block_tables[seg[t]].long()
+        kk = k_cache[bt[idx // BS], :, idx % BS, :].float()
+        vv = v_cache[bt[idx // BS], :, idx % BS, :].float()
+        nb = lo // run if run > 0 else 0
+        if nb:
+            ent = [pool_entry(b, run, BS) for b in range(nb)]
+            pg = bt[torch.tensor([e[0] for e in ent], device=q.device)]
+            off = torch.tensor([e[1] for e in ent], device=q.device)
+            kk = torch.cat([pool_k[pg, :, off, :].float(), kk], 0)
+            vv = torch.cat([pool_v[pg, :, off, :].float(), vv], 0)
+        s = torch.einsum("grd,ngd->grn", q[t].float().view(G, rep, D), kk) * scale
+        if softcap > 0:
+            s = softcap * torch.tanh(s / softcap)
+        o = torch.einsum("grn,ngd->grd", torch.softmax(s, dim=-1), vv).reshape(H, Dv)
+        out[t] = o.to(out.dtype)
+    return out
+
+
+def ssd_recurrence(x, B, C, dt, dt_bias, a_log, skip, state, state_slots, cu_seqlens, seg_start) -> torch.Tensor:
+    """State-space recurrence with a scalar decay per head and token.
+    x [T, H, V], B and C [T, G, N] (already convolved + silu), dt [T, H] raw;
+    per head h of group g: d = softplus(dt + dt_bias), S <- exp(-exp(a_log) d) S
+    + d B x^T, o = S^T C + skip x. state [slots, H, N, V] fp32 is read (unless
+    seg_start == 0) and written back. Everything in fp32; returns o [T, H, V]."""
+    T, H, V = x.shape
+    G = B.shape[1]
+    rep = H // G
+    xf = x.float()
+    Bf = B.float().repeat_interleave(rep, dim=1)
+    Cf = C.float().repeat_interleave(rep, dim=1)
+    d = torch.nn.functional.softplus(dt.float() + dt_bias.float(), threshold=20.0)
+    dec = torch.exp(-torch.exp(a_log.float()) * d)
+    o = torch.empty(T, H, V, dtype=torch.float32, device=x.device)
+    cu, st, sl = cu_seqlens.tolist(), seg_start.tolist(), state_slots.tolist()
+    for b in range(len(sl)):
+        S = state[sl[b]].clone() if st[b] > 0 else torch.zeros_like(state[sl[b]])
+        for t in range(cu[b], cu[b + 1]):
+            S = dec[t].view(H, 1, 1) * S + (d[t].view(H, 1) * Bf[t]).unsqueeze(-1) * xf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hnv,hn->hv", S, Cf[t]) + skip.float().view(H, 1) * xf[t]
+        state[sl[b]] = S
+    return o
+
+
+def gate_group_rmsnorm(o, weight, gate, eps, out_dtype) -> torch.Tensor:
+    """o [T, n_groups, S] fp32 times silu(gate) ([T, n_groups*S] logits), then
+    each group divided by its root mean square, times weight [n_groups*S]."""
+    T, Gn, S = o.shape
+    y = o.float() * torch.nn.functional.silu(gate.float()).view(T, Gn, S)
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+    return (y.reshape(T, Gn * S) * weight.float()).to(out_dtype)
