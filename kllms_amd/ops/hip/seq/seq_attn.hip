@@ -96,14 +96,34 @@ __global__ void qk_norm_store_kernel(T* __restrict__ q, const T* __restrict__ k,
 // at p, plus the first keep_first positions of the sequence. mask_size 0 =
 // plain causal. Visible key number u (0 <= u < nk + p - lo + 1) is position
 // u < nk ? u : lo + u - nk.
-__device__ __forceinline__ void mask_range(int mask_kind, int mask_size, int keep_first, int p, int& lo,
-                                           int& nk) {
+//
+// mask_kind 2: a window of mask_size positions ending at p, and before it one
+// pooled entry per aligned run of ``run`` positions that ends before the window
+// (run u covers u*run .. u*run + run - 1; it is seen when its last position is
+// <= p - mask_size). Visible key u < nk is then pooled run u, not a position.
+__device__ __forceinline__ void mask_range(int mask_kind, int mask_size, int keep_first, int run, int p,
+                                           int& lo, int& nk) {
   lo = 0; nk = 0;
   if (mask_size <= 0) return;
   if (mask_kind == 0) { lo = (p / mask_size) * mask_size; return; }
   lo = max(0, p - mask_size + 1);
-  nk = min(keep_first, lo);
+  nk = mask_kind == 2 ? (run > 0 ? lo / run : 0) : min(keep_first, lo);
 }
+
+// Row of visible key u in the cache it lives in: >= 0 a token row of k_cache /
+// v_cache, <= -2 row -(r + 2) of the pooled caches. A pooled run lives in the
+// page of its last token, counted from the first run that ends in that page.
+__device__ __forceinline__ int visible_row(int u, int nk, int lo, int mask_kind, int run, int PB,
+                                           const int* __restrict__ bt, int G, int g, int BS) {
+  if (u < nk && mask_kind == 2) {
+    const int pg = ((u + 1) * run - 1) / BS;
+    return -(((bt[pg] * G + g) * PB + (u - (pg * BS) / run)) + 2);
+  }
+  const int j = u < nk ? u : lo + (u - nk);
+  return (bt[j / BS] * G + g) * BS + (j % BS);
+}
+
+__device__ __forceinline__ float softcapped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 
 // grid (T, H), one wave per (query row, head). The visible keys in tiles of
 // 64: lane u scores visible key tile*64 + u (q staged in LDS), the tile's weights
@@ -119,6 +139,8 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
                                              const int* __restrict__ token_seg,
                                              const int64_t* __restrict__ positions,
                                              const T* __restrict__ gate, const int* __restrict__ row_map,
+                                             const float* __restrict__ pool_k, const float* __restrict__ pool_v,
+                                             int run, int PB, float softcap,
                                              float scale, int mask_kind, int mask_size, int keep_first,
                                              int sink, int gate_kind,
                                              int H, int G, int D, int Dv, int BS, int bt_stride,
@@ -134,7 +156,7 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
   const int g = h / (H / G);
   const int p = (int)positions[t];
   int lo, nk;
-  mask_range(mask_kind, mask_size, keep_first, p, lo, nk);
+  mask_range(mask_kind, mask_size, keep_first, run, p, lo, nk);
   const int total = nk + (p - lo + 1);
   const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
   const T* qrow = q + (int64_t)t * q_stride + (int64_t)h * D;
@@ -150,12 +172,16 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
     float s = -INFINITY;
     int row = -1;
     if (u < total) {
-      const int j = u < nk ? u : lo + (u - nk);
-      row = (bt[j / BS] * G + g) * BS + (j % BS);
-      const T* kr = k_cache + (int64_t)row * D;
+      row = visible_row(u, nk, lo, mask_kind, run, PB, bt, G, g, BS);
       float d = 0.f;
-      for (int i = 0; i < D; ++i) d += qs[i] * ldf(kr + i);
-      s = d;
+      if (row >= 0) {
+        const T* kr = k_cache + (int64_t)row * D;
+        for (int i = 0; i < D; ++i) d += qs[i] * ldf(kr + i);
+      } else {
+        const float* kr = pool_k + (int64_t)(-(row + 2)) * D;
+        for (int i = 0; i < D; ++i) d += qs[i] * kr[i];
+      }
+      s = softcapped(d, softcap);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float w = u < total ? expf(s - m_new) : 0.f;
@@ -170,11 +196,13 @@ __global__ void attn_blocklocal_paged_kernel(T* __restrict__ out, const T* __res
     for (int i = 0; i < ATTN_MAX_ACC; ++i) acc[i] *= corr;
     for (int jj = 0; jj < n; ++jj) {
       const float pw = ps[jj];
-      const T* vr = v_cache + (int64_t)rows[jj] * Dv;
+      const int rr = rows[jj];
+      const T* vr = v_cache + (int64_t)(rr >= 0 ? rr : 0) * Dv;
+      const float* vp = pool_v + (int64_t)(rr >= 0 ? 0 : -(rr + 2)) * Dv;
 #pragma unroll
       for (int i = 0; i < ATTN_MAX_ACC; ++i) {
         const int d = lane + i * WAVE;
-        if (d < Dv) acc[i] += pw * ldf(vr + d);
+        if (d < Dv) acc[i] += pw * (rr >= 0 ? ldf(vr + d) : vp[d]);
       }
     }
     __syncthreads();
@@ -207,6 +235,7 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, const int* __restrict__ token_seg,
     const int64_t* __restrict__ positions, const T* __restrict__ gate, const int* __restrict__ row_map,
+    const float* __restrict__ pool_k, const float* __restrict__ pool_v, int run, int PB, float softcap,
     float scale, int mask_kind, int mask_size, int keep_first, int sink, int gate_kind, int H, int G, int D,
     int Dv, int BS, int bt_stride, int q_stride, int gate_stride) {
   // The block's waves take the key tiles in turn (tile r*NW + wave in pass
@@ -225,7 +254,7 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
   const int g = h / (H / G);
   const int p = (int)positions[t];
   int lo, nk;
-  mask_range(mask_kind, mask_size, keep_first, p, lo, nk);
+  mask_range(mask_kind, mask_size, keep_first, run, p, lo, nk);
   const int total = nk + (p - lo + 1);
   const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
   const int LPK = D / 8, KPI = WAVE / LPK, kpart = lane % LPK, kgrp = lane / LPK;
@@ -243,20 +272,21 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
     const int base = (r * NW + wave) * WAVE;
     const int n = min(WAVE, total - base);            // <= 0: no tile for this wave in this pass
     const int u = base + lane;
-    const int j = u < nk ? u : lo + (u - nk);
-    rows[lane] = (n > 0 && u < total) ? (bt[j / BS] * G + g) * BS + (j % BS) : -1;
+    rows[lane] = (n > 0 && u < total) ? visible_row(u, nk, lo, mask_kind, run, PB, bt, G, g, BS) : -1;
     __syncthreads();
     for (int it = 0; it * KPI < n; ++it) {
       const int key = it * KPI + kgrp;
       float d = 0.f;
       if (key < n) {
         float kv[8];
-        ld8(k_cache + (int64_t)rows[key] * D + kpart * 8, kv);
+        const int rr = rows[key];
+        if (rr >= 0) ld8(k_cache + (int64_t)rr * D + kpart * 8, kv);
+        else ld8(pool_k + (int64_t)(-(rr + 2)) * D + kpart * 8, kv);
 #pragma unroll
         for (int e = 0; e < 8; ++e) d += qv[e] * kv[e];
       }
       for (int off = 1; off < LPK; off <<= 1) d += __shfl_xor(d, off);
-      if (kpart == 0 && key < n) ps[key] = d;
+      if (kpart == 0 && key < n) ps[key] = softcapped(d, softcap);
     }
     __syncthreads();
     float w = 0.f, corr = 1.f;
@@ -277,7 +307,9 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
       const int key = it * KPV + vgrp;
       if (key < n) {
         float vv[8];
-        ld8(v_cache + (int64_t)rows[key] * Dv + vpart * 8, vv);
+        const int rr = rows[key];
+        if (rr >= 0) ld8(v_cache + (int64_t)rr * Dv + vpart * 8, vv);
+        else ld8(pool_v + (int64_t)(-(rr + 2)) * Dv + vpart * 8, vv);
         const float pw = ps[key];
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[e] += pw * vv[e];
@@ -353,6 +385,87 @@ __global__ void head_gate_v8_kernel(T* __restrict__ out, const T* __restrict__ g
   }
 }
 
+// grid (T, 2), dynamic LDS max(H, G) * D floats. y = 0: the query row — RMS norm
+// over the whole projection (H*D entries, one weight each), rotation of the
+// first 2R entries of every head with entry i paired with i + R
+// (angle = pos * inv_freq[i], fp32), written back in place. y = 1: the same for
+// the key row into k_cache, and the value row into v_cache. The normed row is
+// staged in LDS so that partners are read before anything is overwritten.
+template <typename T>
+__global__ void qk_fullnorm_rope_store_kernel(T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                              const float* __restrict__ wq, const float* __restrict__ wk,
+                                              float eps, const int64_t* __restrict__ positions,
+                                              const float* __restrict__ inv_freq, T* __restrict__ k_cache,
+                                              T* __restrict__ v_cache, const int64_t* __restrict__ slots, int H,
+                                              int G, int D, int Dv, int R, int BS, int q_stride, int k_stride,
+                                              int v_stride) {
+  extern __shared__ float nrow[];
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const bool is_q = blockIdx.y == 0;
+  const int heads = is_q ? H : G;
+  const int n = heads * D;
+  const T* src = is_q ? q + (int64_t)t * q_stride : k + (int64_t)t * k_stride;
+  const float* w = is_q ? wq : wk;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) { const float x = ldf(src + i); nrow[i] = x; ss += x * x; }
+  ss = block_sum(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) nrow[i] *= r * w[i];
+  __syncthreads();
+  const float pos = (float)positions[t];
+  int64_t blk = 0, off = 0;
+  if (!is_q) { const int64_t slot = slots[t]; blk = slot / BS; off = slot % BS; }
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int h = i / D, d = i - h * D;
+    float val = nrow[i];
+    if (d < 2 * R) {
+      const int f = d < R ? d : d - R;
+      float sn, cs;
+      sincosf(pos * inv_freq[f], &sn, &cs);
+      val = d < R ? val * cs - nrow[i + R] * sn : val * cs + nrow[i - R] * sn;
+    }
+    if (is_q) stf(q + (int64_t)t * q_stride + i, val);
+    else stf(k_cache + ((blk * G + h) * BS + off) * D + d, val);
+  }
+  if (!is_q) {
+    for (int i = threadIdx.x; i < G * Dv; i += blockDim.x) {
+      const int g = i / Dv, d = i - g * Dv;
+      v_cache[((blk * G + g) * BS + off) * Dv + d] = v[(int64_t)t * v_stride + i];
+    }
+  }
+}
+
+// grid (T, G): a row whose position ends an aligned run of ``run`` positions
+// writes the fp32 means of the run's cached keys and values into the pooled
+// caches [NB, G, PB, D|Dv]; other rows leave at once. The run's tokens are
+// found through the block table: some may date from earlier steps.
+template <typename T>
+__global__ void pool_kv_update_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                      float* __restrict__ pool_k, float* __restrict__ pool_v,
+                                      const int* __restrict__ block_tables, const int* __restrict__ token_seg,
+                                      const int64_t* __restrict__ positions, int run, int PB, int G, int D,
+                                      int Dv, int BS, int bt_stride) {
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int p = (int)positions[t];
+  if ((p + 1) % run != 0) return;
+  const int b = p / run;
+  const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
+  const int pg = p / BS;
+  const int64_t prow = (int64_t)(bt[pg] * G + g) * PB + (b - (pg * BS) / run);
+  const float inv = 1.0f / (float)run;
+  for (int d = threadIdx.x; d < D + Dv; d += blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < run; ++j) {
+      const int pp = b * run + j;
+      const int64_t row = (int64_t)(bt[pp / BS] * G + g) * BS + (pp % BS);
+      acc += d < D ? ldf(k_cache + row * D + d) : ldf(v_cache + row * Dv + (d - D));
+    }
+    if (d < D) pool_k[prow * D + d] = acc * inv;
+    else pool_v[prow * Dv + (d - D)] = acc * inv;
+  }
+}
+
 #define DISPATCH_T(is_f32, ...)                                  \
   if (is_f32) { typedef float T; __VA_ARGS__ } else { typedef bfraw T; __VA_ARGS__ }
 
@@ -381,6 +494,8 @@ extern "C" void seq_launch_attn_masked_paged(void* out, const void* q, const voi
                                              const void* v_cache, const int* block_tables,
                                              const int* token_seg, const int64_t* positions,
                                              const void* gate, const int* row_map, int n_rows,
+                                             const float* pool_k, const float* pool_v, int run, int PB,
+                                             float softcap,
                                              float scale, int mask_kind, int mask_size, int keep_first,
                                              int sink, int gate_kind, int T_, int H,
                                              int G, int D, int Dv, int BS, int bt_stride, int q_stride,
@@ -390,17 +505,20 @@ extern "C" void seq_launch_attn_masked_paged(void* out, const void* q, const voi
   const int lpk = D / 8, lpv = Dv / 8;
   if (D % 8 == 0 && Dv % 8 == 0 && lpk <= 64 && lpv <= 64 && (lpk & (lpk - 1)) == 0 && (lpv & (lpv - 1)) == 0 &&
       q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out) &&
-      (gate_kind != 2 || (gate_stride % 8 == 0 && aligned16(gate)))) {
+      (gate_kind != 2 || (gate_stride % 8 == 0 && aligned16(gate))) &&
+      (pool_k == nullptr || (aligned16(pool_k) && aligned16(pool_v)))) {
     DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H), dim3(WAVE * ATTN_V8_WAVES), 0, st,
                                           (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
-                                          block_tables, token_seg, positions, (const T*)gate, row_map, scale,
+                                          block_tables, token_seg, positions, (const T*)gate, row_map, pool_k,
+                                          pool_v, run, PB, softcap, scale,
                                           mask_kind, mask_size, keep_first, sink, gate_kind, H, G, D, Dv, BS,
                                           bt_stride, q_stride, gate_stride);)
     return;
   }
   DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(rows, H), dim3(WAVE), lds, st,
                                         (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
-                                        block_tables, token_seg, positions, (const T*)gate, row_map, scale,
+                                        block_tables, token_seg, positions, (const T*)gate, row_map, pool_k,
+                                        pool_v, run, PB, softcap, scale,
                                         mask_kind, mask_size, keep_first, sink, gate_kind,
                                         H, G, D, Dv, BS, bt_stride, q_stride, gate_stride);)
 }
@@ -417,4 +535,28 @@ extern "C" void seq_launch_head_gate(void* out, const void* gate, int T_, int H,
   const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(head_gate_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,
                                         (const T*)gate, n, H, Dv, gate_stride);)
+}
+
+extern "C" void seq_launch_qk_fullnorm_rope_store(void* q, const void* k, const void* v, const float* wq,
+                                                  const float* wk, float eps, const int64_t* positions,
+                                                  const float* inv_freq, void* k_cache, void* v_cache,
+                                                  const int64_t* slots, int T_, int H, int G, int D, int Dv,
+                                                  int R, int BS, int q_stride, int k_stride, int v_stride,
+                                                  int is_f32, hipStream_t st) {
+  const int heads = H > G ? H : G;
+  const size_t lds = (size_t)heads * D * sizeof(float);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(qk_fullnorm_rope_store_kernel<T>, dim3(T_, k != nullptr ? 2 : 1),
+                                        dim3(256), lds, st, (T*)q, (const T*)k, (const T*)v, wq, wk, eps,
+                                        positions, inv_freq, (T*)k_cache, (T*)v_cache, slots, H, G, D, Dv, R, BS,
+                                        q_stride, k_stride, v_stride);)
+}
+
+extern "C" void seq_launch_pool_kv_update(const void* k_cache, const void* v_cache, float* pool_k, float* pool_v,
+                                          const int* block_tables, const int* token_seg,
+                                          const int64_t* positions, int run, int PB, int T_, int G, int D, int Dv,
+                                          int BS, int bt_stride, int is_f32, hipStream_t st) {
+  const int threads = D + Dv > 128 ? 256 : (D + Dv > 64 ? 128 : 64);
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(pool_kv_update_kernel<T>, dim3(T_, G), dim3(threads), 0, st,
+                                        (const T*)k_cache, (const T*)v_cache, pool_k, pool_v, block_tables,
+                                        token_seg, positions, run, PB, G, D, Dv, BS, bt_stride);)
 }

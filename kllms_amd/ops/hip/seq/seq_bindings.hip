@@ -30,8 +30,21 @@ void seq_launch_rope_pairs_store(void*, const void*, const void*, const int64_t*
                                  const int64_t*, void*, int, int, int, int, int, int, int, int, int, int, int,
                                  hipStream_t);
 void seq_launch_attn_masked_paged(void*, const void*, const void*, const void*, const int*, const int*,
-                                  const int64_t*, const void*, const int*, int, float, int, int, int, int, int,
+                                  const int64_t*, const void*, const int*, int, const float*, const float*, int,
+                                  int, float, float, int, int, int, int, int,
                                   int, int, int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_qk_fullnorm_rope_store(void*, const void*, const void*, const float*, const float*, float,
+                                       const int64_t*, const float*, void*, void*, const int64_t*, int, int, int,
+                                       int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_pool_kv_update(const void*, const void*, float*, float*, const int*, const int*, const int64_t*,
+                               int, int, int, int, int, int, int, int, int, hipStream_t);
+void seq_launch_ln_residual_mix(float*, const float*, const void*, const float*, float*, float*, const float*, int,
+                                int64_t, int, int, float, int, hipStream_t);
+void seq_launch_ln_canon(void*, const float*, const float*, const float*, const float*, float*, int64_t,
+                         const int*, const int*, const int*, const int*, int, int, int, int, int, hipStream_t);
+void seq_launch_ssd_recurrence(float*, const void*, const void*, const void*, const void*, const float*,
+                               const float*, const float*, float*, float*, float*, const int*, const int*,
+                               const int*, int, int, int, int, int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_qk_norm_store(void*, const void*, const void*, const float*, const float*, float, void*, void*,
                               const int64_t*, int, int, int, int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_embed_bigram(float*, const int64_t*, const void*, const void*, float, int, int, int, int*,
@@ -59,7 +72,7 @@ void seq_launch_linear_attn_decay(float*, const void*, const void*, const void*,
                                   const int*, const int*, const int*, int, int, int, int, int, int, int, int,
                                   int, hipStream_t);
 void seq_launch_causal_conv_silu(void*, const void*, const float*, void*, const int*, const int*, const int*,
-                                 const int*, int, int, int, int, int, int, hipStream_t);
+                                 const int*, const float*, int, int, int, int, int, int, hipStream_t);
 void seq_launch_gated_delta_rule(float*, const void*, const void*, const void*, const void*, const void*,
                                  const float*, const float*, float*, float*, float*, float*, float*, float*,
                                  const int*, const int*, const int*, int, int, int, int, int, int, int, int, int,
@@ -305,7 +318,8 @@ void rope_pairs_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::
 void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache, torch::Tensor v_cache,
                        torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
                        torch::Tensor gate, double scale, int64_t mask_kind, int64_t mask_size,
-                       int64_t keep_first, bool sink, torch::Tensor row_map) {
+                       int64_t keep_first, bool sink, torch::Tensor row_map, torch::Tensor pool_k,
+                       torch::Tensor pool_v, int64_t run, double softcap) {
   CHECK_ACT(q); CHECK_ROWS3(q); CHECK_SAME(out, q); CHECK_SAME(k_cache, q); CHECK_SAME(v_cache, q);
   CHECK_I32C(block_tables); CHECK_I32C(token_seg); CHECK_I64C(positions);
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && k_cache.is_cuda() && v_cache.is_cuda() &&
@@ -313,7 +327,19 @@ void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
   const int T = q.size(0), H = q.size(1), D = q.size(2);
   const int G = k_cache.size(1), BS = k_cache.size(2), Dv = v_cache.size(3);
   TORCH_CHECK(k_cache.size(3) == D && H % G == 0 && Dv <= 512 && mask_size >= 0 && keep_first >= 0);
-  TORCH_CHECK(mask_kind == 0 || mask_kind == 1, "mask_kind: 0 = aligned blocks, 1 = sliding window");
+  TORCH_CHECK(mask_kind >= 0 && mask_kind <= 2,
+              "mask_kind: 0 = aligned blocks, 1 = sliding window, 2 = sliding window + pooled runs");
+  // pooled caches [NB, G, ceil(BS / run), D|Dv] fp32, used by mask_kind 2 with run > 0
+  const bool pooled = mask_kind == 2 && run > 0 && mask_size > 0;
+  int PB = 0;
+  if (pooled) {
+    CHECK_F32C(pool_k); CHECK_F32C(pool_v);
+    PB = (BS + (int)run - 1) / (int)run;
+    TORCH_CHECK(pool_k.dim() == 4 && pool_v.dim() == 4 && pool_k.size(0) == k_cache.size(0) &&
+                pool_v.size(0) == k_cache.size(0) && pool_k.size(1) == G && pool_v.size(1) == G &&
+                pool_k.size(2) == PB && pool_v.size(2) == PB && pool_k.size(3) == D && pool_v.size(3) == Dv);
+  }
+  TORCH_CHECK(softcap >= 0.0);
   TORCH_CHECK(out.numel() == (int64_t)T * H * Dv && token_seg.numel() == T && positions.numel() == T);
   int gate_kind = 0;
   if (gate.numel() > 0) {
@@ -328,7 +354,9 @@ void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
                                block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
                                positions.data_ptr<int64_t>(), gate_kind ? gate.data_ptr() : nullptr,
                                mapped ? row_map.data_ptr<int>() : nullptr, (int)row_map.numel(),
-                               (float)scale, (int)mask_kind, (int)mask_size, (int)keep_first, sink ? 1 : 0,
+                               pooled ? pool_k.data_ptr<float>() : nullptr,
+                               pooled ? pool_v.data_ptr<float>() : nullptr, pooled ? (int)run : 0, PB,
+                               (float)softcap, (float)scale, (int)mask_kind, (int)mask_size, (int)keep_first, sink ? 1 : 0,
                                gate_kind, T, H, G, D, Dv, BS,
                                (int)block_tables.stride(0), (int)q.stride(0),
                                gate_kind ? (int)gate.stride(0) : 0, f32flag(q), cur_stream());
@@ -414,8 +442,11 @@ void linear_attn_decay(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch:
 }
 
 void causal_conv_silu(torch::Tensor y, torch::Tensor x, torch::Tensor w, torch::Tensor conv_state,
-                      torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start, torch::Tensor token_seg) {
+                      torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start, torch::Tensor token_seg,
+                      torch::Tensor bias) {
   CHECK_ACT(x); CHECK_ROWS2(x); CHECK_SAME(y, x); CHECK_SAME(conv_state, x); CHECK_F32C(w); CHECK_I32C(token_seg);
+  const bool has_bias = bias.numel() > 0;
+  if (has_bias) { CHECK_F32C(bias); TORCH_CHECK(bias.numel() == x.size(1)); }
   check_segments(slots, cu, seg_start, conv_state);
   // w: taps-major [K, C], last row = the current token's tap
   TORCH_CHECK(w.dim() == 2);
@@ -427,7 +458,8 @@ void causal_conv_silu(torch::Tensor y, torch::Tensor x, torch::Tensor w, torch::
   if (T == 0 || B == 0) return;
   seq_launch_causal_conv_silu(y.data_ptr(), x.data_ptr(), w.data_ptr<float>(), conv_state.data_ptr(),
                               slots.data_ptr<int>(), cu.data_ptr<int>(), seg_start.data_ptr<int>(),
-                              token_seg.data_ptr<int>(), T, B, C, K, (int)x.stride(0), f32flag(x), cur_stream());
+                              token_seg.data_ptr<int>(), has_bias ? bias.data_ptr<float>() : nullptr, T, B, C, K,
+                              (int)x.stride(0), f32flag(x), cur_stream());
 }
 
 void gated_delta_rule(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor beta,
@@ -537,7 +569,8 @@ void head_rmsnorm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor w, torc
   const int T = o.size(0), H = o.size(1), S = (int)o.size(2) - (ext ? 1 : 0);
   TORCH_CHECK(S >= 1 && out.numel() == (int64_t)T * H * S);
   TORCH_CHECK(w.numel() == (int64_t)H * S && gate.size(0) == T && gate.size(1) == (int64_t)H * S);
-  TORCH_CHECK(gate_act == 0 || gate_act == 1, "gate_act: 0 = sigmoid, 1 = silu");
+  TORCH_CHECK(gate_act >= 0 && gate_act <= 2, "gate_act: 0 = sigmoid, 1 = silu, 2 = silu before the norm");
+  TORCH_CHECK(gate_act != 2 || !ext);
   if (ext) { CHECK_F32C(mt); TORCH_CHECK(mt.numel() == (int64_t)T * H); }
   if (T == 0) return;
   seq_launch_head_rmsnorm_gate(out.data_ptr(), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(),
@@ -687,6 +720,139 @@ void mlstm_recurrence(torch::Tensor o, torch::Tensor q, torch::Tensor k, torch::
                               (int)q.stride(0), (int)k.stride(0), (int)v.stride(0), f32flag(q), cur_stream());
 }
 
+// ---- layer-normed sublayers with an input convolution, depth-weighted stream ----
+
+// a / w_post empty: x_out = x_in. streams empty: no depth average.
+void ln_residual_mix(torch::Tensor x_out, torch::Tensor x_in, torch::Tensor a, torch::Tensor w_post,
+                     torch::Tensor stats, torch::Tensor streams, torch::Tensor dwa, int64_t n_prev, double eps) {
+  CHECK_F32C(x_out); CHECK_F32C(x_in); CHECK_F32C(stats);
+  TORCH_CHECK(x_in.dim() == 2 && x_out.sizes() == x_in.sizes());
+  const int T = x_in.size(0), W = x_in.size(1);
+  TORCH_CHECK(W >= 1 && W <= 16384 && stats.numel() == 2 * (int64_t)T);
+  const bool has_a = a.numel() > 0, mix = streams.numel() > 0;
+  if (has_a) {
+    CHECK_ACT(a); CHECK_F32C(w_post);
+    TORCH_CHECK(a.is_contiguous() && a.dim() == 2 && a.size(0) == T && a.size(1) == W && w_post.numel() == W);
+  }
+  if (mix) {
+    CHECK_F32C(streams); CHECK_F32C(dwa);
+    TORCH_CHECK(streams.dim() == 3 && streams.size(1) == T && streams.size(2) == W && n_prev >= 0 &&
+                n_prev < streams.size(0) && dwa.numel() == n_prev + 1);
+  }
+  if (T == 0) return;
+  seq_launch_ln_residual_mix(x_out.data_ptr<float>(), x_in.data_ptr<float>(), has_a ? a.data_ptr() : nullptr,
+                             has_a ? w_post.data_ptr<float>() : nullptr, stats.data_ptr<float>(),
+                             mix ? streams.data_ptr<float>() : nullptr, mix ? dwa.data_ptr<float>() : nullptr,
+                             (int)n_prev, (int64_t)T * W, T, W, (float)eps, has_a ? f32flag(a) : 1, cur_stream());
+}
+
+// cw empty: the norm alone. hist: [slots, K-1, W] fp32 view (rows packed, free slot stride).
+void ln_canon(torch::Tensor out, torch::Tensor x, torch::Tensor stats, torch::Tensor w, torch::Tensor cw,
+              torch::Tensor hist, torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start,
+              torch::Tensor token_seg) {
+  CHECK_ACT(out); CHECK_F32C(x); CHECK_F32C(stats); CHECK_F32C(w);
+  TORCH_CHECK(x.dim() == 2 && out.is_contiguous() && out.numel() == x.numel());
+  const int T = x.size(0), W = x.size(1);
+  TORCH_CHECK(w.numel() == W && stats.numel() == 2 * (int64_t)T);
+  int K = 0, B = 0;
+  int64_t hist_stride = 0;
+  if (cw.numel() > 0) {
+    CHECK_F32C(cw); CHECK_I32C(token_seg);
+    check_segments(slots, cu, seg_start, T);
+    TORCH_CHECK(cw.dim() == 2 && cw.size(1) == W && token_seg.numel() == T);
+    K = cw.size(0);
+    B = slots.numel();
+    TORCH_CHECK(K >= 1 && K <= 16, "1..16 convolution taps supported");
+    if (K > 1) {
+      TORCH_CHECK(hist.is_cuda() && hist.scalar_type() == at::kFloat && hist.dim() == 3 && hist.size(1) == K - 1 &&
+                  hist.size(2) == W && hist.stride(2) == 1 && hist.stride(1) == W);
+      hist_stride = hist.stride(0);
+    }
+  }
+  if (T == 0) return;
+  seq_launch_ln_canon(out.data_ptr(), x.data_ptr<float>(), stats.data_ptr<float>(), w.data_ptr<float>(),
+                      K ? cw.data_ptr<float>() : nullptr, K > 1 ? hist.data_ptr<float>() : nullptr, hist_stride,
+                      K ? slots.data_ptr<int>() : nullptr, K ? cu.data_ptr<int>() : nullptr,
+                      K ? seg_start.data_ptr<int>() : nullptr, K ? token_seg.data_ptr<int>() : nullptr, T, B, W, K,
+                      f32flag(out), cur_stream());
+}
+
+// k empty: the layer reads another layer's cache, only q is normed and rotated
+void qk_fullnorm_rope_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor wq, torch::Tensor wk,
+                            double eps, torch::Tensor positions, torch::Tensor inv_freq, torch::Tensor k_cache,
+                            torch::Tensor v_cache, torch::Tensor slots) {
+  CHECK_ACT(q); CHECK_ROWS3(q); CHECK_F32C(wq); CHECK_I64C(positions); CHECK_F32C(inv_freq);
+  const int T = q.size(0), H = q.size(1), D = q.size(2), R = inv_freq.numel();
+  TORCH_CHECK(wq.numel() == (int64_t)H * D && positions.numel() == T && 2 * R <= D);
+  const bool has_k = k.numel() > 0;
+  int G = 0, Dv = 0, BS = 1;
+  if (has_k) {
+    CHECK_ROWS3(k); CHECK_ROWS3(v); CHECK_SAME(k, q); CHECK_SAME(v, q); CHECK_SAME(k_cache, q);
+    CHECK_SAME(v_cache, q); CHECK_F32C(wk); CHECK_I64C(slots);
+    TORCH_CHECK(k.is_cuda() && v.is_cuda() && k_cache.is_cuda() && v_cache.is_cuda() && k_cache.is_contiguous() &&
+                v_cache.is_contiguous() && k_cache.dim() == 4 && v_cache.dim() == 4);
+    G = k.size(1); Dv = v.size(2); BS = k_cache.size(2);
+    TORCH_CHECK(k.size(0) == T && k.size(2) == D && v.size(0) == T && v.size(1) == G);
+    TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == D && v_cache.size(1) == G && v_cache.size(2) == BS &&
+                v_cache.size(3) == Dv && v_cache.size(0) == k_cache.size(0));
+    TORCH_CHECK(wk.numel() == (int64_t)G * D && slots.numel() == T);
+  }
+  TORCH_CHECK((int64_t)(H > G ? H : G) * D <= 15360, "projection too wide for the norm kernel's staging");
+  if (T == 0) return;
+  seq_launch_qk_fullnorm_rope_store(q.data_ptr(), has_k ? k.data_ptr() : nullptr, has_k ? v.data_ptr() : nullptr,
+                                    wq.data_ptr<float>(), has_k ? wk.data_ptr<float>() : nullptr, (float)eps,
+                                    positions.data_ptr<int64_t>(), inv_freq.data_ptr<float>(),
+                                    has_k ? k_cache.data_ptr() : nullptr, has_k ? v_cache.data_ptr() : nullptr,
+                                    has_k ? slots.data_ptr<int64_t>() : nullptr, T, H, G, D, Dv, R, BS,
+                                    (int)q.stride(0), has_k ? (int)k.stride(0) : 0, has_k ? (int)v.stride(0) : 0,
+                                    f32flag(q), cur_stream());
+}
+
+void pool_kv_update(torch::Tensor k_cache, torch::Tensor v_cache, torch::Tensor pool_k, torch::Tensor pool_v,
+                    torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions, int64_t run) {
+  CHECK_ACT(k_cache); CHECK_SAME(v_cache, k_cache); CHECK_F32C(pool_k); CHECK_F32C(pool_v);
+  CHECK_I32C(block_tables); CHECK_I32C(token_seg); CHECK_I64C(positions);
+  TORCH_CHECK(v_cache.is_cuda() && k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 4 &&
+              v_cache.dim() == 4 && pool_k.dim() == 4 && pool_v.dim() == 4 && block_tables.dim() == 2 && run >= 1);
+  const int G = k_cache.size(1), BS = k_cache.size(2), D = k_cache.size(3), Dv = v_cache.size(3);
+  const int PB = (BS + (int)run - 1) / (int)run, T = positions.numel();
+  TORCH_CHECK(v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G && v_cache.size(2) == BS);
+  TORCH_CHECK(pool_k.size(0) == k_cache.size(0) && pool_v.size(0) == k_cache.size(0) && pool_k.size(1) == G &&
+              pool_v.size(1) == G && pool_k.size(2) == PB && pool_v.size(2) == PB && pool_k.size(3) == D &&
+              pool_v.size(3) == Dv && token_seg.numel() == T);
+  if (T == 0) return;
+  seq_launch_pool_kv_update(k_cache.data_ptr(), v_cache.data_ptr(), pool_k.data_ptr<float>(),
+                            pool_v.data_ptr<float>(), block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
+                            positions.data_ptr<int64_t>(), (int)run, PB, T, G, D, Dv, BS,
+                            (int)block_tables.stride(0), f32flag(k_cache), cur_stream());
+}
+
+// x [T, H, V], B / C [T, G, N] row views, dt [T, H] row view; state [slots, H, N, V] fp32
+void ssd_recurrence(torch::Tensor o, torch::Tensor x, torch::Tensor Bm, torch::Tensor Cm, torch::Tensor dt,
+                    torch::Tensor dt_bias, torch::Tensor a_log, torch::Tensor skip, torch::Tensor state,
+                    torch::Tensor slots, torch::Tensor cu, torch::Tensor seg_start) {
+  CHECK_F32C(o); CHECK_ACT(x); CHECK_ROWS3(x); CHECK_ROWS3(Bm); CHECK_ROWS3(Cm); CHECK_ROWS2(dt);
+  CHECK_SAME(Bm, x); CHECK_SAME(Cm, x); CHECK_SAME(dt, x);
+  CHECK_F32C(dt_bias); CHECK_F32C(a_log); CHECK_F32C(skip); CHECK_F32C(state);
+  check_segments(slots, cu, seg_start, state);
+  const int T = x.size(0), H = x.size(1), V = x.size(2), G = Bm.size(1), N = Bm.size(2), B = slots.numel();
+  TORCH_CHECK(Bm.is_cuda() && Cm.is_cuda() && dt.is_cuda() && Bm.size(0) == T && Cm.size(0) == T &&
+              Cm.size(1) == G && Cm.size(2) == N && dt.size(0) == T && dt.size(1) == H && G >= 1 && H % G == 0);
+  TORCH_CHECK(N <= 256, "state size above 256 is not supported by the recurrence kernel");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == N && state.size(3) == V);
+  TORCH_CHECK(dt_bias.numel() == H && a_log.numel() == H && skip.numel() == H && o.numel() == (int64_t)T * H * V);
+  if (T == 0 || B == 0) return;
+  auto opt = torch::dtype(torch::kFloat).device(x.device());
+  auto packed = torch::empty({(int64_t)T, (int64_t)H * (2 * N + V)}, opt);
+  auto dec = torch::empty({(int64_t)T, (int64_t)H}, opt);
+  seq_launch_ssd_recurrence(o.data_ptr<float>(), x.data_ptr(), Bm.data_ptr(), Cm.data_ptr(), dt.data_ptr(),
+                            dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), skip.data_ptr<float>(),
+                            packed.data_ptr<float>(), dec.data_ptr<float>(), state.data_ptr<float>(),
+                            slots.data_ptr<int>(), cu.data_ptr<int>(), seg_start.data_ptr<int>(), T, B, H, G, N, V,
+                            (int)x.stride(0), (int)Bm.stride(0), (int)Cm.stride(0), (int)dt.stride(0), f32flag(x),
+                            cur_stream());
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_rmsnorm", &embed_rmsnorm);
   m.def("rmsnorm_cast", &rmsnorm_cast);
@@ -716,4 +882,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("linear_attn_decay", &linear_attn_decay);
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("gated_delta_rule", &gated_delta_rule);
+  m.def("ln_residual_mix", &ln_residual_mix);
+  m.def("ln_canon", &ln_canon);
+  m.def("qk_fullnorm_rope_store", &qk_fullnorm_rope_store);
+  m.def("pool_kv_update", &pool_kv_update);
+  m.def("ssd_recurrence", &ssd_recurrence);
 }

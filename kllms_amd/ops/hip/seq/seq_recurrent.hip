@@ -68,8 +68,11 @@ __global__ void linear_prep_v8_kernel(float* __restrict__ pk, const T* __restric
 template <int DMAX, int NS>
 __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
     float* __restrict__ o, const float* __restrict__ pk, const float* __restrict__ decay,
+    const float* __restrict__ decay_t, const float* __restrict__ skip,
     float* __restrict__ state, const int* __restrict__ slots, const int* __restrict__ cu,
     const int* __restrict__ seg_start, int H, int D, int V) {
+  // decay_t != nullptr: one decay per (token, head) [T, H] instead of decay[h];
+  // skip != nullptr: o += skip[h] * v (a direct path from the value to the output)
   constexpr int TB = 4;                                   // tokens per pipeline stage
   constexpr int DR = DMAX / NS, COLS = WAVE / NS;         // state rows / columns per lane group
   constexpr int PER = (2 * DMAX + WAVE - 1) / WAVE;       // q|k elements staged per lane
@@ -84,7 +87,8 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
   const bool fresh = seg_start[b] == 0;
 #pragma unroll
   for (int d = 0; d < DR; ++d) S[d] = (!fresh && live && d0 + d < D) ? sp[(int64_t)(d0 + d) * V] : 0.f;
-  const float dec = decay[h];
+  const float dec = decay_t ? 0.f : decay[h];
+  const float skp = skip ? skip[h] : 0.f;
   if (t1 - t0 == 1) {
     // decode: one row. No pipeline — stage q|k once (zeros above D), update, read out.
     const float* row = pk + ((int64_t)t0 * H + h) * W;
@@ -94,17 +98,18 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
       buf[i] = d < D ? row[i < DMAX ? d : D + d] : 0.f;
     }
     const float vj = live ? row[2 * D + j] : 0.f;
+    const float dc = decay_t ? decay_t[(int64_t)t0 * H + h] : dec;
     __syncthreads();
     float acc = 0.f;
 #pragma unroll
     for (int d = 0; d < DR; ++d) {
-      S[d] = dec * S[d] + buf[DMAX + d0 + d] * vj;
+      S[d] = dc * S[d] + buf[DMAX + d0 + d] * vj;
       acc += S[d] * buf[d0 + d];
     }
 #pragma unroll
     for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off);
     if (live) {
-      if (grp == 0) o[((int64_t)t0 * H + h) * V + j] = acc;
+      if (grp == 0) o[((int64_t)t0 * H + h) * V + j] = acc + skp * vj;
 #pragma unroll
       for (int d = 0; d < DR; ++d) if (d0 + d < D) sp[(int64_t)(d0 + d) * V] = S[d];
     }
@@ -117,7 +122,7 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
   __syncthreads();
   // software pipeline over groups of TB tokens: the next group's operands are
   // in flight while this group's tokens are computed one after the other
-  float pre[TB][PER], vpre[TB];
+  float pre[TB][PER], vpre[TB], dpre[TB];
   auto fetch = [&](int tg) {
 #pragma unroll
     for (int u = 0; u < TB; ++u) {
@@ -130,12 +135,13 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
         pre[u][r] = (on && i < 2 * D) ? row[i] : 0.f;
       }
       vpre[u] = (on && live) ? row[2 * D + j] : 0.f;
+      dpre[u] = (on && decay_t) ? decay_t[(int64_t)t * H + h] : dec;
     }
   };
   if (t0 < t1) fetch(t0);
   int flip = 0;
   for (int tg = t0; tg < t1; tg += TB, flip ^= 1) {
-    float vj[TB];
+    float vj[TB], dc[TB];
 #pragma unroll
     for (int u = 0; u < TB; ++u) {
 #pragma unroll
@@ -144,6 +150,7 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
         if (i < 2 * D) qk[flip][u][i < D ? i : DMAX + (i - D)] = pre[u][r];
       }
       vj[u] = vpre[u];
+      dc[u] = dpre[u];
     }
     __syncthreads();    // double-buffered: one barrier per group
     if (tg + TB < t1) fetch(tg + TB);
@@ -154,12 +161,12 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
         float acc = 0.f;
 #pragma unroll
         for (int d = 0; d < DR; ++d) {
-          S[d] = dec * S[d] + buf[DMAX + d0 + d] * vj[u];
+          S[d] = dc[u] * S[d] + buf[DMAX + d0 + d] * vj[u];
           acc += S[d] * buf[d0 + d];
         }
 #pragma unroll
         for (int off = COLS; off < WAVE; off <<= 1) acc += __shfl_xor(acc, off);
-        if (live && grp == 0) o[((int64_t)(tg + u) * H + h) * V + j] = acc;
+        if (live && grp == 0) o[((int64_t)(tg + u) * H + h) * V + j] = acc + skp * vj[u];
       }
     }
   }
@@ -170,7 +177,7 @@ __global__ void __launch_bounds__(WAVE) linear_attn_decay_kernel(
 }
 
 // ---- short causal convolution + silu ----------------------------------------
-// y[t,c] = silu(sum_j w[j,c] * x[t - (K-1-j), c]) (weights taps-major [K, C],
+// y[t,c] = silu(bias[c] + sum_j w[j,c] * x[t - (K-1-j), c]) (bias optional; weights taps-major [K, C],
 // last tap = current token); inputs before the segment
 // come from conv_state [slot, K-1, C] (oldest first), zeros for a fresh sequence.
 template <typename T>
@@ -178,7 +185,7 @@ __global__ void causal_conv_silu_kernel(T* __restrict__ y, const T* __restrict__
                                         const float* __restrict__ w, const T* __restrict__ conv_state,
                                         const int* __restrict__ slots, const int* __restrict__ cu,
                                         const int* __restrict__ seg_start, const int* __restrict__ token_seg,
-                                        int64_t n, int C, int K, int x_stride) {
+                                        const float* __restrict__ bias, int64_t n, int C, int K, int x_stride) {
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n;
        idx += (int64_t)gridDim.x * blockDim.x) {
     const int t = (int)(idx / C), c = (int)(idx - (int64_t)t * C);
@@ -186,7 +193,7 @@ __global__ void causal_conv_silu_kernel(T* __restrict__ y, const T* __restrict__
     const int i = t - cu[b];
     const bool fresh = seg_start[b] == 0;
     const T* hist = conv_state + (int64_t)slots[b] * (K - 1) * C;
-    float acc = 0.f;
+    float acc = bias ? bias[c] : 0.f;
     for (int j = 0; j < K; ++j) {
       const int src = i - (K - 1 - j);
       float xv;
@@ -204,7 +211,8 @@ __global__ void causal_conv_silu_v8_kernel(T* __restrict__ y, const T* __restric
                                            const float* __restrict__ w, const T* __restrict__ conv_state,
                                            const int* __restrict__ slots, const int* __restrict__ cu,
                                            const int* __restrict__ seg_start,
-                                           const int* __restrict__ token_seg, int64_t n8, int C, int K,
+                                           const int* __restrict__ token_seg,
+                                           const float* __restrict__ bias, int64_t n8, int C, int K,
                                            int x_stride) {
   const int C8 = C / 8;
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n8;
@@ -215,6 +223,7 @@ __global__ void causal_conv_silu_v8_kernel(T* __restrict__ y, const T* __restric
     const bool fresh = seg_start[b] == 0;
     const T* hist = conv_state + (int64_t)slots[b] * (K - 1) * C;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (bias) ld8(bias + c, acc);
     for (int j = 0; j < K; ++j) {
       const int src = i - (K - 1 - j);
       float xv[8], wv[8];
@@ -477,26 +486,68 @@ extern "C" void seq_launch_linear_attn_decay(float* o, const void* q, const void
   const int ns = pick_split(B, H, V);
   DISPATCH_NS(ns, DISPATCH_D(D, hipLaunchKernelGGL((linear_attn_decay_kernel<DMAX, NS>),
                                                    dim3(B, H, (V + WAVE / NS - 1) / (WAVE / NS)), dim3(WAVE), 0,
-                                                   st, o, packed, decay, state, slots, cu, seg_start, H, D, V);))
+                                                   st, o, packed, decay, nullptr, nullptr, state, slots, cu,
+                                                   seg_start, H, D, V);))
+}
+
+// ---- state-space recurrence with a scalar decay per head and token ---------------
+// d = softplus(dt + dt_bias); S <- exp(-exp(A_h) d) S + (d B_g) x_h^T; o = S^T C_g + D_h x_h
+// A parallel pre-pass (one wave per (token, head)) writes the recurrence's
+// operands in fp32 in the packed layout of linear_attn_decay_kernel —
+// [C_g (N) | d B_g (N) | x_h (V)] — and the decay per (token, head); the
+// recurrence itself is that kernel with a per-token decay and the skip term.
+template <typename T>
+__global__ void ssd_prep_kernel(float* __restrict__ pk, float* __restrict__ dec, const T* __restrict__ x,
+                                const T* __restrict__ Bm, const T* __restrict__ Cm, const T* __restrict__ dt,
+                                const float* __restrict__ dt_bias, const float* __restrict__ a_log, int H, int G,
+                                int N, int V, int x_stride, int b_stride, int c_stride, int dt_stride) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (H / G);
+  const float d = softplus_exact(ldf(dt + t * dt_stride + h) + dt_bias[h]);
+  if (lane == 0) dec[t * H + h] = expf(-expf(a_log[h]) * d);
+  float* row = pk + (t * H + h) * (2 * N + V);
+  const T* cr = Cm + t * c_stride + (int64_t)g * N;
+  const T* br = Bm + t * b_stride + (int64_t)g * N;
+  const T* xr = x + t * x_stride + (int64_t)h * V;
+  for (int i = lane; i < N; i += WAVE) { row[i] = ldf(cr + i); row[N + i] = d * ldf(br + i); }
+  for (int i = lane; i < V; i += WAVE) row[2 * N + i] = ldf(xr + i);
+}
+
+extern "C" void seq_launch_ssd_recurrence(float* o, const void* x, const void* Bm, const void* Cm, const void* dt,
+                                          const float* dt_bias, const float* a_log, const float* skip,
+                                          float* packed, float* dec, float* state, const int* slots,
+                                          const int* cu, const int* seg_start, int T_, int B, int H, int G, int N,
+                                          int V, int x_stride, int b_stride, int c_stride, int dt_stride,
+                                          int is_f32, hipStream_t st) {
+  DISPATCH_T(is_f32, hipLaunchKernelGGL(ssd_prep_kernel<T>, dim3(T_, H), dim3(WAVE), 0, st, packed, dec,
+                                        (const T*)x, (const T*)Bm, (const T*)Cm, (const T*)dt, dt_bias, a_log, H,
+                                        G, N, V, x_stride, b_stride, c_stride, dt_stride);)
+  const int ns = pick_split(B, H, V);
+  const int D = N;
+  DISPATCH_NS(ns, DISPATCH_D(D, hipLaunchKernelGGL((linear_attn_decay_kernel<DMAX, NS>),
+                                                   dim3(B, H, (V + WAVE / NS - 1) / (WAVE / NS)), dim3(WAVE), 0,
+                                                   st, o, packed, nullptr, dec, skip, state, slots, cu, seg_start,
+                                                   H, N, V);))
 }
 
 extern "C" void seq_launch_causal_conv_silu(void* y, const void* x, const float* w, void* conv_state,
                                             const int* slots, const int* cu, const int* seg_start,
-                                            const int* token_seg, int T_, int B, int C, int K, int x_stride,
-                                            int is_f32, hipStream_t st) {
+                                            const int* token_seg, const float* bias, int T_, int B, int C, int K,
+                                            int x_stride, int is_f32, hipStream_t st) {
   const int64_t n = (int64_t)T_ * C;
   const int grid = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   const int grid2 = (int)(((int64_t)B * C + 255) / 256);
   const bool v8 = C % 8 == 0 && x_stride % 8 == 0 && aligned16(y) && aligned16(x) && aligned16(conv_state) &&
-                  aligned16(w);
+                  aligned16(w) && (bias == nullptr || aligned16(bias));
   const int g8 = (int)((n / 8 + 255) / 256 < 16384 ? (n / 8 + 255) / 256 : 16384);
   DISPATCH_T(is_f32,
              if (v8) hipLaunchKernelGGL(causal_conv_silu_v8_kernel<T>, dim3(g8), dim3(256), 0, st, (T*)y,
                                         (const T*)x, w, (const T*)conv_state, slots, cu, seg_start, token_seg,
-                                        n / 8, C, K, x_stride);
+                                        bias, n / 8, C, K, x_stride);
              else hipLaunchKernelGGL(causal_conv_silu_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)y, (const T*)x,
-                                w, (const T*)conv_state, slots, cu, seg_start, token_seg, n, C, K, x_stride);
-             hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(grid2), dim3(256), 0, st, (const T*)x,
+                                w, (const T*)conv_state, slots, cu, seg_start, token_seg, bias, n, C, K, x_stride);
+             if (K > 1) hipLaunchKernelGGL(conv_state_update_kernel<T>, dim3(grid2), dim3(256), 0, st, (const T*)x,
                                 (T*)conv_state, slots, cu, seg_start, B, C, K, x_stride);)
 }
 

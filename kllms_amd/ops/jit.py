@@ -36,7 +36,7 @@ EXTENSIONS = {
         "dir": os.path.join(HIP_DIR, "seq"),
         # the dense MFMA prefill kernel is shared with _C (one source, two modules)
         "kernels": ["seq_norm.hip", "seq_attn.hip", "seq_recurrent.hip", "seq_parallel.hip", "seq_gated.hip",
-                    "seq_latent.hip", "../attn_prefill.hip"],
+                    "seq_latent.hip", "seq_stream.hip", "../attn_prefill.hip"],
         "bindings": ["seq_bindings.hip"],
         "headers": ["seq_common.h"],
     },
