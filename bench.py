@@ -29,7 +29,7 @@ and scheduler, other ranks follow in lockstep (parallel/serve.py).
 
 ``--compare-families`` is a separate, single-GPU measurement: prefill and
 decode token throughput of the listed-layer families (Zutalix, Medilix,
-Mitunex; ``--families`` picks) beside
+Mitunex, Pironex; ``--families`` picks) beside
 the dense Llama stack of the same width / depth / heads / ff, straight through
 LLMEngine.generate (random-init weights, synthetic token ids). It prints its
 own JSON line and leaves the default workload untouched.
@@ -212,7 +212,7 @@ def main():
                     help="prefill/decode tok/s of the hybrid families beside the dense Llama stack of equal shape")
     ap.add_argument("--families", type=str, default="llama,zutalix,medilix",
                     help="--compare-families: model families to time, in order "
-                         "(llama, zutalix, medilix, mitunex)")
+                         "(llama, zutalix, medilix, mitunex, pironex)")
     ap.add_argument("--sizes", type=str, default="1b-l6,8b-l6", help="--compare-families: preset size suffixes")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)

@@ -385,7 +385,7 @@ __global__ void head_gate_v8_kernel(T* __restrict__ out, const T* __restrict__ g
   }
 }
 
-// grid (T, 2), dynamic LDS max(H, G) * D floats. y = 0: the query row — RMS norm
+// grid (T, 2), dynamic LDS (max(H, G) * D + 2R) floats. y = 0: the query row — RMS norm
 // over the whole projection (H*D entries, one weight each), rotation of the
 // first 2R entries of every head with entry i paired with i + R
 // (angle = pos * inv_freq[i], fp32), written back in place. y = 1: the same for
@@ -399,7 +399,7 @@ __global__ void qk_fullnorm_rope_store_kernel(T* __restrict__ q, const T* __rest
                                               T* __restrict__ v_cache, const int64_t* __restrict__ slots, int H,
                                               int G, int D, int Dv, int R, int BS, int q_stride, int k_stride,
                                               int v_stride) {
-  extern __shared__ float nrow[];
+  extern __shared__ float nrow[];          // the normed row | cos [R] | sin [R]
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const bool is_q = blockIdx.y == 0;
@@ -412,8 +412,11 @@ __global__ void qk_fullnorm_rope_store_kernel(T* __restrict__ q, const T* __rest
   ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)n + eps);
   for (int i = threadIdx.x; i < n; i += blockDim.x) nrow[i] *= r * w[i];
-  __syncthreads();
   const float pos = (float)positions[t];
+  float* cs_t = nrow + n;
+  float* sn_t = cs_t + R;
+  for (int i = threadIdx.x; i < R; i += blockDim.x) sincosf(pos * inv_freq[i], &sn_t[i], &cs_t[i]);
+  __syncthreads();
   int64_t blk = 0, off = 0;
   if (!is_q) { const int64_t slot = slots[t]; blk = slot / BS; off = slot % BS; }
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -421,8 +424,7 @@ __global__ void qk_fullnorm_rope_store_kernel(T* __restrict__ q, const T* __rest
     float val = nrow[i];
     if (d < 2 * R) {
       const int f = d < R ? d : d - R;
-      float sn, cs;
-      sincosf(pos * inv_freq[f], &sn, &cs);
+      const float sn = sn_t[f], cs = cs_t[f];
       val = d < R ? val * cs - nrow[i + R] * sn : val * cs + nrow[i - R] * sn;
     }
     if (is_q) stf(q + (int64_t)t * q_stride + i, val);
@@ -463,6 +465,53 @@ __global__ void pool_kv_update_kernel(const T* __restrict__ k_cache, const T* __
     }
     if (d < D) pool_k[prow * D + d] = acc * inv;
     else pool_v[prow * Dv + (d - D)] = acc * inv;
+  }
+}
+
+// The same with 16-byte loads (D and Dv multiples of 8, (D + Dv) / 8 <= 256):
+// LPP lanes cover one token's key and value row, the block's 256 / LPP lane
+// groups take the run's tokens in turn, and their partial sums meet in LDS.
+template <typename T>
+__global__ void __launch_bounds__(256) pool_kv_update_v8_kernel(
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache, float* __restrict__ pool_k,
+    float* __restrict__ pool_v, const int* __restrict__ block_tables, const int* __restrict__ token_seg,
+    const int64_t* __restrict__ positions, int run, int PB, int G, int D, int Dv, int BS, int bt_stride) {
+  __shared__ float red[256 * 8];
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int p = (int)positions[t];
+  if ((p + 1) % run != 0) return;
+  const int b = p / run;
+  const int* bt = block_tables + (int64_t)token_seg[t] * bt_stride;
+  const int pg = p / BS;
+  const int64_t prow = (int64_t)(bt[pg] * G + g) * PB + (b - (pg * BS) / run);
+  const int LPP = (D + Dv) / 8, NPG = 256 / LPP;
+  const int dl = threadIdx.x % LPP, grp = threadIdx.x / LPP;
+  const int d0 = dl * 8;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (grp < NPG) {
+    for (int j = grp; j < run; j += NPG) {
+      const int pp = b * run + j;
+      const int64_t row = (int64_t)(bt[pp / BS] * G + g) * BS + (pp % BS);
+      float v[8];
+      if (d0 < D) ld8(k_cache + row * D + d0, v);
+      else ld8(v_cache + row * Dv + (d0 - D), v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) red[threadIdx.x * 8 + e] = acc[e];
+  __syncthreads();
+  if (grp == 0) {
+    for (int g2 = 1; g2 < NPG; ++g2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += red[(g2 * LPP + dl) * 8 + e];
+    }
+    const float inv = 1.0f / (float)run;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= inv;
+    if (d0 < D) st8(pool_k + prow * D + d0, acc);
+    else st8(pool_v + prow * Dv + (d0 - D), acc);
   }
 }
 
@@ -544,7 +593,7 @@ extern "C" void seq_launch_qk_fullnorm_rope_store(void* q, const void* k, const 
                                                   int R, int BS, int q_stride, int k_stride, int v_stride,
                                                   int is_f32, hipStream_t st) {
   const int heads = H > G ? H : G;
-  const size_t lds = (size_t)heads * D * sizeof(float);
+  const size_t lds = ((size_t)heads * D + 2 * R) * sizeof(float);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(qk_fullnorm_rope_store_kernel<T>, dim3(T_, k != nullptr ? 2 : 1),
                                         dim3(256), lds, st, (T*)q, (const T*)k, (const T*)v, wq, wk, eps,
                                         positions, inv_freq, (T*)k_cache, (T*)v_cache, slots, H, G, D, Dv, R, BS,
@@ -555,6 +604,13 @@ extern "C" void seq_launch_pool_kv_update(const void* k_cache, const void* v_cac
                                           const int* block_tables, const int* token_seg,
                                           const int64_t* positions, int run, int PB, int T_, int G, int D, int Dv,
                                           int BS, int bt_stride, int is_f32, hipStream_t st) {
+  if (D % 8 == 0 && Dv % 8 == 0 && (D + Dv) / 8 <= 256 && aligned16(k_cache) && aligned16(v_cache) &&
+      aligned16(pool_k) && aligned16(pool_v)) {
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(pool_kv_update_v8_kernel<T>, dim3(T_, G), dim3(256), 0, st,
+                                          (const T*)k_cache, (const T*)v_cache, pool_k, pool_v, block_tables,
+                                          token_seg, positions, run, PB, G, D, Dv, BS, bt_stride);)
+    return;
+  }
   const int threads = D + Dv > 128 ? 256 : (D + Dv > 64 ? 128 : 64);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(pool_kv_update_kernel<T>, dim3(T_, G), dim3(threads), 0, st,
                                         (const T*)k_cache, (const T*)v_cache, pool_k, pool_v, block_tables,
