@@ -305,7 +305,8 @@ def attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, s
                                  gate if gate is not None else _none(q), scale, int(mask_kind), int(mask_size),
                                  int(keep_first), bool(sink),
                                  row_map if row_map is not None else _none(q, torch.int32),
-                                 _none(q, torch.float32), _none(q, torch.float32), 0, 0.0)
+                                 _none(q, torch.float32), _none(q, torch.float32), 0, 0.0,
+                                 _none(q, torch.float32), _none(q, torch.float32))
         return out
     assert row_map is None and out is None
     return torch_ref.attn_masked_paged(q, k_cache, v_cache, block_tables, token_seg, positions, scale,
@@ -713,17 +714,29 @@ def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, po
 
 
 def attn_window_pool_paged(q, k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, scale,
-                           softcap, mask_size, run):
+                           softcap, mask_size, run, key_splits: int = 0):
     """Sliding-window attention over the paged cache with the pooled entries
     of the runs that lie wholly before the window, soft-capped scores; prompt
-    portions, decoded tokens and mixes alike."""
+    portions, decoded tokens and mixes alike. ``key_splits`` (GPU): workgroups
+    that share one (row, head)'s keys, merged by a second kernel; 0 = as many
+    as fill the chip for this step (few rows, long windows), 1 = none."""
     if _gpu(q):
         out = torch.empty((q.shape[0], q.shape[1], v_cache.shape[3]), dtype=q.dtype, device=q.device)
         f = _none(q, torch.float32)
         has = run > 0
+        # steps of few rows: a (row, head)'s key tiles are shared out over several workgroups.
+        # An upper bound of the visible keys, from the mask or the block table's width
+        T, H = q.shape[0], q.shape[1]
+        ctx = block_tables.shape[1] * k_cache.shape[2]
+        reach = min(ctx, mask_size + (ctx // run if has else 0)) if mask_size > 0 else ctx
+        tiles = (reach + 63) // 64
+        ns = key_splits or max(1, min((tiles + 3) // 4, 512 // max(1, T * H), 64))
+        part_o = torch.empty((T, H, ns, v_cache.shape[3]), dtype=torch.float32, device=q.device) if ns > 1 else f
+        part_ml = torch.empty((T, H, ns, 2), dtype=torch.float32, device=q.device) if ns > 1 else f
         _seq().attn_masked_paged(out, q, k_cache, v_cache, block_tables, token_seg, positions, _none(q),
                                  scale, 2, int(mask_size), 0, False, _none(q, torch.int32),
-                                 pool_k if has else f, pool_v if has else f, int(run), float(softcap))
+                                 pool_k if has else f, pool_v if has else f, int(run), float(softcap),
+                                 part_o, part_ml)
         return out
     return torch_ref.attn_window_pool_paged(q, k_cache, v_cache, pool_k, pool_v, block_tables, token_seg,
                                             positions, scale, softcap, mask_size, run)

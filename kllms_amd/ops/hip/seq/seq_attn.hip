@@ -236,8 +236,14 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
     const int* __restrict__ block_tables, const int* __restrict__ token_seg,
     const int64_t* __restrict__ positions, const T* __restrict__ gate, const int* __restrict__ row_map,
     const float* __restrict__ pool_k, const float* __restrict__ pool_v, int run, int PB, float softcap,
+    float* __restrict__ part_o, float* __restrict__ part_ml,
     float scale, int mask_kind, int mask_size, int keep_first, int sink, int gate_kind, int H, int G, int D,
     int Dv, int BS, int bt_stride, int q_stride, int gate_stride) {
+  // gridDim.z > 1 (steps of few rows): the workgroups of one (row, head) take
+  // contiguous shares of its key tiles and leave unnormalised partial results
+  // (sums relative to the share's maximum, that maximum and the sum of weights)
+  // in part_o [T, H, Z, Dv] / part_ml [T, H, Z, 2]; attn_split_merge_kernel
+  // combines them in a fixed order.
   // The block's waves take the key tiles in turn (tile r*NW + wave in pass
   // r), each with its own running max / sum / accumulator; the partial
   // results are merged through LDS at the end. Every wave runs every pass —
@@ -265,12 +271,15 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
   for (int e = 0; e < 8; ++e) qv[e] *= scale;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   // the sink is one more key of score 0 without a value, held by wave 0
-  const bool sunk = sink && wave == 0;
+  const bool sunk = sink && wave == 0 && blockIdx.z == 0;
   float m = sunk ? 0.f : -INFINITY, l = sunk ? 1.f : 0.f;
   const int ntiles = (total + WAVE - 1) / WAVE;
-  for (int r = 0; r * NW < ntiles; ++r) {
-    const int base = (r * NW + wave) * WAVE;
-    const int n = min(WAVE, total - base);            // <= 0: no tile for this wave in this pass
+  const int per_share = (ntiles + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int tile0 = (int)blockIdx.z * per_share, tile1 = min(ntiles, tile0 + per_share);
+  for (int r = 0; tile0 + r * NW < tile1; ++r) {
+    const int tile = tile0 + r * NW + wave;
+    const int base = tile * WAVE;
+    const int n = tile < tile1 ? min(WAVE, total - base) : 0;   // 0: no tile for this wave in this pass
     const int u = base + lane;
     rows[lane] = (n > 0 && u < total) ? visible_row(u, nk, lo, mask_kind, run, PB, bt, G, g, BS) : -1;
     __syncthreads();
@@ -340,6 +349,12 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
 #pragma unroll
       for (int e = 0; e < 8; ++e) o8[e] += part_acc[w2][vpart * 8 + e] * f;
     }
+    if (gridDim.z > 1) {
+      const int64_t pz = ((int64_t)t * H + h) * gridDim.z + blockIdx.z;
+      if (vpart == 0) { part_ml[2 * pz] = M; part_ml[2 * pz + 1] = L; }
+      st8(part_o + pz * Dv + vpart * 8, o8);
+      return;
+    }
     float gsc = 1.0f / L;
     if (gate_kind == 1) gsc *= sigmoid_exact(ldf(gate + (int64_t)t * gate_stride + h));
 #pragma unroll
@@ -351,6 +366,39 @@ __global__ void __launch_bounds__(WAVE * ATTN_V8_WAVES) attn_blocklocal_paged_v8
       for (int e = 0; e < 8; ++e) o8[e] *= sigmoid_exact(g8[e]);
     }
     st8(out + ((int64_t)t * H + h) * Dv + vpart * 8, o8);
+  }
+}
+
+// Merge of the key shares of one (row, head): grid (T, H), one thread per 8
+// output dims. out = sum_z o_z e^(m_z - M) / sum_z l_z e^(m_z - M), M = max m_z,
+// summed over z in order; a share that saw no key (l = 0) counts for nothing.
+template <typename T>
+__global__ void attn_split_merge_kernel(T* __restrict__ out, const float* __restrict__ part_o,
+                                        const float* __restrict__ part_ml, int H, int Dv, int nsplit) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int64_t base = ((int64_t)t * H + h) * nsplit;
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) if (part_ml[2 * (base + z) + 1] > 0.f) M = fmaxf(M, part_ml[2 * (base + z)]);
+  float L = 0.f;
+  for (int z = 0; z < nsplit; ++z) {
+    const float lz = part_ml[2 * (base + z) + 1];
+    if (lz > 0.f) L += lz * expf(part_ml[2 * (base + z)] - M);
+  }
+  const float inv = 1.0f / L;
+  for (int d = threadIdx.x * 8; d < Dv; d += blockDim.x * 8) {
+    float o8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, v[8];
+    for (int z = 0; z < nsplit; ++z) {
+      const float lz = part_ml[2 * (base + z) + 1];
+      if (lz > 0.f) {
+        const float f = expf(part_ml[2 * (base + z)] - M);
+        ld8(part_o + (base + z) * Dv + d, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o8[e] += v[e] * f;
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o8[e] *= inv;
+    st8(out + ((int64_t)t * H + h) * Dv + d, o8);
   }
 }
 
@@ -544,7 +592,7 @@ extern "C" void seq_launch_attn_masked_paged(void* out, const void* q, const voi
                                              const int* token_seg, const int64_t* positions,
                                              const void* gate, const int* row_map, int n_rows,
                                              const float* pool_k, const float* pool_v, int run, int PB,
-                                             float softcap,
+                                             float softcap, int nsplit, float* part_o, float* part_ml,
                                              float scale, int mask_kind, int mask_size, int keep_first,
                                              int sink, int gate_kind, int T_, int H,
                                              int G, int D, int Dv, int BS, int bt_stride, int q_stride,
@@ -556,12 +604,19 @@ extern "C" void seq_launch_attn_masked_paged(void* out, const void* q, const voi
       q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && aligned16(out) &&
       (gate_kind != 2 || (gate_stride % 8 == 0 && aligned16(gate))) &&
       (pool_k == nullptr || (aligned16(pool_k) && aligned16(pool_v)))) {
-    DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H), dim3(WAVE * ATTN_V8_WAVES), 0, st,
+    // key shares only for plain launches: every row, no gate
+    const int ns = (nsplit > 1 && row_map == nullptr && gate_kind == 0 && part_o != nullptr) ? nsplit : 1;
+    DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_v8_kernel<T>, dim3(rows, H, ns), dim3(WAVE * ATTN_V8_WAVES), 0, st,
                                           (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache,
                                           block_tables, token_seg, positions, (const T*)gate, row_map, pool_k,
-                                          pool_v, run, PB, softcap, scale,
+                                          pool_v, run, PB, softcap, part_o, part_ml, scale,
                                           mask_kind, mask_size, keep_first, sink, gate_kind, H, G, D, Dv, BS,
                                           bt_stride, q_stride, gate_stride);)
+    if (ns > 1) {
+      const int threads = Dv / 8 > WAVE ? 2 * WAVE : WAVE;
+      DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_split_merge_kernel<T>, dim3(rows, H), dim3(threads), 0, st,
+                                            (T*)out, part_o, part_ml, H, Dv, ns);)
+    }
     return;
   }
   DISPATCH_T(is_f32, hipLaunchKernelGGL(attn_blocklocal_paged_kernel<T>, dim3(rows, H), dim3(WAVE), lds, st,

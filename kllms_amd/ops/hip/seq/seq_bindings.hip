@@ -31,7 +31,7 @@ void seq_launch_rope_pairs_store(void*, const void*, const void*, const int64_t*
                                  hipStream_t);
 void seq_launch_attn_masked_paged(void*, const void*, const void*, const void*, const int*, const int*,
                                   const int64_t*, const void*, const int*, int, const float*, const float*, int,
-                                  int, float, float, int, int, int, int, int,
+                                  int, float, int, float*, float*, float, int, int, int, int, int,
                                   int, int, int, int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_qk_fullnorm_rope_store(void*, const void*, const void*, const float*, const float*, float,
                                        const int64_t*, const float*, void*, void*, const int64_t*, int, int, int,
@@ -319,7 +319,8 @@ void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
                        torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions,
                        torch::Tensor gate, double scale, int64_t mask_kind, int64_t mask_size,
                        int64_t keep_first, bool sink, torch::Tensor row_map, torch::Tensor pool_k,
-                       torch::Tensor pool_v, int64_t run, double softcap) {
+                       torch::Tensor pool_v, int64_t run, double softcap, torch::Tensor part_o,
+                       torch::Tensor part_ml) {
   CHECK_ACT(q); CHECK_ROWS3(q); CHECK_SAME(out, q); CHECK_SAME(k_cache, q); CHECK_SAME(v_cache, q);
   CHECK_I32C(block_tables); CHECK_I32C(token_seg); CHECK_I64C(positions);
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && k_cache.is_cuda() && v_cache.is_cuda() &&
@@ -340,6 +341,14 @@ void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
                 pool_k.size(2) == PB && pool_v.size(2) == PB && pool_k.size(3) == D && pool_v.size(3) == Dv);
   }
   TORCH_CHECK(softcap >= 0.0);
+  // key shares: part_o [T, H, Z, Dv], part_ml [T, H, Z, 2] fp32 scratch; empty = one workgroup per (row, head)
+  int nsplit = 1;
+  if (part_o.numel() > 0) {
+    CHECK_F32C(part_o); CHECK_F32C(part_ml);
+    TORCH_CHECK(part_o.dim() == 4 && part_o.size(0) == T && part_o.size(1) == H && part_o.size(3) == Dv &&
+                part_ml.numel() == (int64_t)T * H * part_o.size(2) * 2 && part_o.size(2) <= 64);
+    nsplit = part_o.size(2);
+  }
   TORCH_CHECK(out.numel() == (int64_t)T * H * Dv && token_seg.numel() == T && positions.numel() == T);
   int gate_kind = 0;
   if (gate.numel() > 0) {
@@ -356,7 +365,8 @@ void attn_masked_paged(torch::Tensor out, torch::Tensor q, torch::Tensor k_cache
                                mapped ? row_map.data_ptr<int>() : nullptr, (int)row_map.numel(),
                                pooled ? pool_k.data_ptr<float>() : nullptr,
                                pooled ? pool_v.data_ptr<float>() : nullptr, pooled ? (int)run : 0, PB,
-                               (float)softcap, (float)scale, (int)mask_kind, (int)mask_size, (int)keep_first, sink ? 1 : 0,
+                               (float)softcap, nsplit, nsplit > 1 ? part_o.data_ptr<float>() : nullptr,
+                               nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, (float)scale, (int)mask_kind, (int)mask_size, (int)keep_first, sink ? 1 : 0,
                                gate_kind, T, H, G, D, Dv, BS,
                                (int)block_tables.stride(0), (int)q.stride(0),
                                gate_kind ? (int)gate.stride(0) : 0, f32flag(q), cur_stream());

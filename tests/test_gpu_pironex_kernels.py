@@ -166,9 +166,11 @@ def test_pooled_runs_update_and_attention(dtype, G, D, Dv, BS, run):
         ts = i32([s for s, _ in rows])
         ps = torch.tensor([p for _, p in rows], device=DEV)
         q = rnd(len(rows), H, D, dtype=dtype, seed=size, std=1.5)
-        o1 = ops.attn_window_pool_paged(q, kc, vc, pk1, pv1, bt, ts, ps, 0.3, cap, size, run)
         o2 = torch_ref.attn_window_pool_paged(q, kc, vc, pk2, pv2, bt, ts, ps, 0.3, cap, size, run)
-        close(o1, o2, dtype)
+        # one workgroup per (row, head), and the keys shared out over 2 and 5 (more shares than key tiles)
+        for splits in (1, 0, 2, 5):
+            o1 = ops.attn_window_pool_paged(q, kc, vc, pk1, pv1, bt, ts, ps, 0.3, cap, size, run, key_splits=splits)
+            close(o1, o2, dtype)
         # without pooling the far tokens are simply gone
         o3 = ops.attn_window_pool_paged(q, kc, vc, None, None, bt, ts, ps, 0.3, cap, size, 0)
         o4 = torch_ref.attn_window_pool_paged(q, kc, vc, None, None, bt, ts, ps, 0.3, cap, size, 0)
