@@ -480,6 +480,23 @@ class PoolWindowAttention(nn.Module):
         return LayerCacheSpec(kv=kv if self.own_kv else None, kv_of=sp.kv_from,
                               pool=kv + (sp.pool,) if sp.pool > 0 and sp.mask_size > 0 else None)
 
+    @staticmethod
+    def _run_ends(batch, run: int) -> Optional[torch.Tensor]:
+        """Rows of the step whose position ends a run (int32, possibly empty),
+        when the step was built on the host; None = not known, look at every
+        row. Most decode steps complete no run and skip the pooling launch."""
+        if batch.host_segs is None or batch.plans is None:
+            return None
+        key = ("run_ends", run)
+        if key not in batch.plans:
+            rows, row0 = [], 0
+            for start, n in batch.host_segs:
+                first = (-(start + 1)) % run            # first offset with (start + offset + 1) % run == 0
+                rows.extend(range(row0 + first, row0 + n, run))
+                row0 += n
+            batch.plans[key] = torch.tensor(rows, dtype=torch.int32, device=batch.positions.device)
+        return batch.plans[key]
+
     def forward(self, h: torch.Tensor, batch, st: LayerState) -> torch.Tensor:
         sp = self.spec
         T = h.shape[0]
@@ -494,8 +511,10 @@ class PoolWindowAttention(nn.Module):
                                    st.k, st.v, batch.slot_mapping)
         run = sp.pool if st.pool_k is not None else 0
         if run:
-            ops.pool_kv_update(st.k, st.v, st.pool_k, st.pool_v, batch.block_tables, batch.token_seg,
-                               batch.positions, run)
+            rows = self._run_ends(batch, run)
+            if rows is None or rows.numel():
+                ops.pool_kv_update(st.k, st.v, st.pool_k, st.pool_v, batch.block_tables, batch.token_seg,
+                                   batch.positions, run, rows)
         att = ops.attn_window_pool_paged(q, st.k, st.v, st.pool_k, st.pool_v, batch.block_tables, batch.token_seg,
                                          batch.positions, sp.scale, sp.softcap, sp.mask_size, run)
         return F.linear(att.reshape(T, -1), self.o_proj)

@@ -703,14 +703,17 @@ def qk_fullnorm_rope_store(q, k, v, wq, wk, eps, positions, inv_freq, k_cache, v
     torch_ref.qk_fullnorm_rope_store(q, k, v, wq, wk, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
 
 
-def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run: int) -> None:
+def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run: int,
+                   row_map=None) -> None:
     """Means of the cached keys / values of every aligned run of ``run``
     positions that one of this step's rows completes, into the fp32 pooled
-    caches."""
+    caches. ``row_map`` (int32): the rows to look at, when the caller knows
+    which rows end a run; None = every row."""
     if _gpu(k_cache):
-        _seq().pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, int(run))
+        _seq().pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, int(run),
+                              row_map if row_map is not None else _none(k_cache, torch.int32))
         return
-    torch_ref.pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run)
+    torch_ref.pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run, row_map)
 
 
 def attn_window_pool_paged(q, k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, scale,

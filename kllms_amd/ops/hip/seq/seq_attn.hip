@@ -486,17 +486,18 @@ __global__ void qk_fullnorm_rope_store_kernel(T* __restrict__ q, const T* __rest
   }
 }
 
-// grid (T, G): a row whose position ends an aligned run of ``run`` positions
+// grid (rows, G): a row whose position ends an aligned run of ``run`` positions
 // writes the fp32 means of the run's cached keys and values into the pooled
-// caches [NB, G, PB, D|Dv]; other rows leave at once. The run's tokens are
+// caches [NB, G, PB, D|Dv]; other rows leave at once. row_map (optional): the
+// rows to look at — the host knows which rows of a prompt portion end a run. The run's tokens are
 // found through the block table: some may date from earlier steps.
 template <typename T>
 __global__ void pool_kv_update_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                       float* __restrict__ pool_k, float* __restrict__ pool_v,
                                       const int* __restrict__ block_tables, const int* __restrict__ token_seg,
-                                      const int64_t* __restrict__ positions, int run, int PB, int G, int D,
-                                      int Dv, int BS, int bt_stride) {
-  const int t = blockIdx.x, g = blockIdx.y;
+                                      const int64_t* __restrict__ positions, const int* __restrict__ row_map,
+                                      int run, int PB, int G, int D, int Dv, int BS, int bt_stride) {
+  const int t = row_map ? row_map[blockIdx.x] : blockIdx.x, g = blockIdx.y;
   const int p = (int)positions[t];
   if ((p + 1) % run != 0) return;
   const int b = p / run;
@@ -523,9 +524,10 @@ template <typename T>
 __global__ void __launch_bounds__(256) pool_kv_update_v8_kernel(
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, float* __restrict__ pool_k,
     float* __restrict__ pool_v, const int* __restrict__ block_tables, const int* __restrict__ token_seg,
-    const int64_t* __restrict__ positions, int run, int PB, int G, int D, int Dv, int BS, int bt_stride) {
+    const int64_t* __restrict__ positions, const int* __restrict__ row_map, int run, int PB, int G, int D,
+    int Dv, int BS, int bt_stride) {
   __shared__ float red[256 * 8];
-  const int t = blockIdx.x, g = blockIdx.y;
+  const int t = row_map ? row_map[blockIdx.x] : blockIdx.x, g = blockIdx.y;
   const int p = (int)positions[t];
   if ((p + 1) % run != 0) return;
   const int b = p / run;
@@ -657,17 +659,18 @@ extern "C" void seq_launch_qk_fullnorm_rope_store(void* q, const void* k, const 
 
 extern "C" void seq_launch_pool_kv_update(const void* k_cache, const void* v_cache, float* pool_k, float* pool_v,
                                           const int* block_tables, const int* token_seg,
-                                          const int64_t* positions, int run, int PB, int T_, int G, int D, int Dv,
-                                          int BS, int bt_stride, int is_f32, hipStream_t st) {
+                                          const int64_t* positions, const int* row_map, int run, int PB, int T_,
+                                          int G, int D, int Dv, int BS, int bt_stride, int is_f32,
+                                          hipStream_t st) {
   if (D % 8 == 0 && Dv % 8 == 0 && (D + Dv) / 8 <= 256 && aligned16(k_cache) && aligned16(v_cache) &&
       aligned16(pool_k) && aligned16(pool_v)) {
     DISPATCH_T(is_f32, hipLaunchKernelGGL(pool_kv_update_v8_kernel<T>, dim3(T_, G), dim3(256), 0, st,
                                           (const T*)k_cache, (const T*)v_cache, pool_k, pool_v, block_tables,
-                                          token_seg, positions, run, PB, G, D, Dv, BS, bt_stride);)
+                                          token_seg, positions, row_map, run, PB, G, D, Dv, BS, bt_stride);)
     return;
   }
   const int threads = D + Dv > 128 ? 256 : (D + Dv > 64 ? 128 : 64);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(pool_kv_update_kernel<T>, dim3(T_, G), dim3(threads), 0, st,
                                         (const T*)k_cache, (const T*)v_cache, pool_k, pool_v, block_tables,
-                                        token_seg, positions, run, PB, G, D, Dv, BS, bt_stride);)
+                                        token_seg, positions, row_map, run, PB, G, D, Dv, BS, bt_stride);)
 }

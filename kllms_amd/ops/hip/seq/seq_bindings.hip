@@ -37,7 +37,7 @@ void seq_launch_qk_fullnorm_rope_store(void*, const void*, const void*, const fl
                                        const int64_t*, const float*, void*, void*, const int64_t*, int, int, int,
                                        int, int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_pool_kv_update(const void*, const void*, float*, float*, const int*, const int*, const int64_t*,
-                               int, int, int, int, int, int, int, int, int, hipStream_t);
+                               const int*, int, int, int, int, int, int, int, int, int, hipStream_t);
 void seq_launch_ln_residual_mix(float*, const float*, const void*, const float*, float*, float*, const float*, int,
                                 int64_t, int, int, float, int, hipStream_t);
 void seq_launch_ln_canon(void*, const float*, const float*, const float*, const float*, float*, int64_t,
@@ -819,21 +819,28 @@ void qk_fullnorm_rope_store(torch::Tensor q, torch::Tensor k, torch::Tensor v, t
 }
 
 void pool_kv_update(torch::Tensor k_cache, torch::Tensor v_cache, torch::Tensor pool_k, torch::Tensor pool_v,
-                    torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions, int64_t run) {
+                    torch::Tensor block_tables, torch::Tensor token_seg, torch::Tensor positions, int64_t run,
+                    torch::Tensor row_map) {
   CHECK_ACT(k_cache); CHECK_SAME(v_cache, k_cache); CHECK_F32C(pool_k); CHECK_F32C(pool_v);
   CHECK_I32C(block_tables); CHECK_I32C(token_seg); CHECK_I64C(positions);
   TORCH_CHECK(v_cache.is_cuda() && k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 4 &&
               v_cache.dim() == 4 && pool_k.dim() == 4 && pool_v.dim() == 4 && block_tables.dim() == 2 && run >= 1);
   const int G = k_cache.size(1), BS = k_cache.size(2), D = k_cache.size(3), Dv = v_cache.size(3);
-  const int PB = (BS + (int)run - 1) / (int)run, T = positions.numel();
+  const int PB = (BS + (int)run - 1) / (int)run;
+  // row_map: the rows (of this step) to look at; empty = all
+  const bool mapped = row_map.numel() > 0;
+  if (mapped) { CHECK_I32C(row_map); TORCH_CHECK(row_map.numel() <= positions.numel()); }
+  TORCH_CHECK(token_seg.numel() == positions.numel());
+  const int T = mapped ? (int)row_map.numel() : (int)positions.numel();
   TORCH_CHECK(v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G && v_cache.size(2) == BS);
   TORCH_CHECK(pool_k.size(0) == k_cache.size(0) && pool_v.size(0) == k_cache.size(0) && pool_k.size(1) == G &&
               pool_v.size(1) == G && pool_k.size(2) == PB && pool_v.size(2) == PB && pool_k.size(3) == D &&
-              pool_v.size(3) == Dv && token_seg.numel() == T);
+              pool_v.size(3) == Dv);
   if (T == 0) return;
   seq_launch_pool_kv_update(k_cache.data_ptr(), v_cache.data_ptr(), pool_k.data_ptr<float>(),
                             pool_v.data_ptr<float>(), block_tables.data_ptr<int>(), token_seg.data_ptr<int>(),
-                            positions.data_ptr<int64_t>(), (int)run, PB, T, G, D, Dv, BS,
+                            positions.data_ptr<int64_t>(), mapped ? row_map.data_ptr<int>() : nullptr, (int)run, PB,
+                            T, G, D, Dv, BS,
                             (int)block_tables.stride(0), f32flag(k_cache), cur_stream());
 }
 

@@ -892,13 +892,15 @@ def pool_entry(b: int, run: int, BS: int):
     return pg, b - (pg * BS) // run
 
 
-def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run: int) -> None:
-    """For every row whose position ends an aligned run of ``run`` positions:
-    the fp32 means of the run's cached keys and values go to pool_k / pool_v
-    [NB, G, ceil(BS / run), D|Dv]."""
+def pool_kv_update(k_cache, v_cache, pool_k, pool_v, block_tables, token_seg, positions, run: int,
+                   row_map=None) -> None:
+    """For every row (of row_map, or of the step) whose position ends an
+    aligned run of ``run`` positions: the fp32 means of the run's cached keys
+    and values go to pool_k / pool_v [NB, G, ceil(BS / run), D|Dv]."""
     BS = k_cache.shape[2]
     pos, seg = positions.tolist(), token_seg.tolist()
-    for t, p in enumerate(pos):
+    for t in (range(len(pos)) if row_map is None else row_map.tolist()):
+        p = pos[t]
         if (p + 1) % run:
             continue
         b = p // run

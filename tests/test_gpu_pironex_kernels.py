@@ -158,6 +158,14 @@ def test_pooled_runs_update_and_attention(dtype, G, D, Dv, BS, run):
     torch_ref.pool_kv_update(kc, vc, pk2, pv2, bt, tseg, pos, run)
     close(pk1, pk2, torch.float32, scale=8)
     close(pv1, pv2, torch.float32, scale=8)
+    # the same through a list of the rows that end a run (in any order), and an untouched cache for other rows
+    ends = [t for t in range(n_seq * ctx) if (t % ctx + 1) % run == 0]
+    pk3, pv3 = torch.full_like(pk1, 7.0), torch.full_like(pv1, -7.0)
+    ops.pool_kv_update(kc, vc, pk3, pv3, bt, tseg, pos, run, i32(ends[::-1]))
+    assert torch.equal(pk3, pk1) and torch.equal(pv3, pv1)
+    pk3.fill_(7.0)
+    ops.pool_kv_update(kc, vc, pk3, pv3, bt, tseg, pos, run, i32([run - 1, run]))     # one row ends a run, one does not
+    assert int((pk3 != 7.0).sum()) == G * D
     # attention rows: a portion in the middle, single rows, the first rows, edges of window and runs
     for size, cap in [(37, 0.0), (run, 5.0), (1, 0.0), (200, 3.0)]:
         rows = [(0, 0), (0, 1), (1, size - 1), (1, size), (2, size + run - 2), (2, size + run - 1), (2, size + run),
