@@ -366,7 +366,7 @@ def linear_attn_decay(q, k, v, decay, state, state_slots, cu_seqlens, seg_start)
 def gated_rmsnorm(o, weight, gate, eps, out_dtype):
     if _gpu(o):
         out = torch.empty((o.shape[0], o.shape[1] * o.shape[2]), dtype=out_dtype, device=o.device)
-        _seq().gated_rmsnorm(out, o, weight, gate, eps)
+        _seq().gated_rmsnorm(out, o, weight, gate, eps, False)
         return out
     return torch_ref.gated_rmsnorm(o, weight, gate, eps, out_dtype)
 
@@ -759,6 +759,6 @@ def gate_group_rmsnorm(o, weight, gate, eps, out_dtype):
     """(o * silu(gate)) RMS-normed in groups, times weight: o [T, groups, S] fp32."""
     if _gpu(o):
         out = torch.empty((o.shape[0], o.shape[1] * o.shape[2]), dtype=out_dtype, device=o.device)
-        _seq().head_rmsnorm_gate(out, o, weight, gate, eps, 2, _none(o, torch.float32))
+        _seq().gated_rmsnorm(out, o, weight, gate, eps, True)
         return out
     return torch_ref.gate_group_rmsnorm(o, weight, gate, eps, out_dtype)

@@ -23,7 +23,7 @@ void seq_launch_rmsnorm_cast(void*, const float*, const float*, int, int, float,
 void seq_launch_sandwich_residual(float*, const void*, const void*, const float*, const float*, const float*,
                                   const float*, void*, int, int, float, int, hipStream_t);
 void seq_launch_gated_rmsnorm(void*, const float*, const float*, const void*, int, int, int, int, float, int,
-                              hipStream_t);
+                              int, hipStream_t);
 void seq_launch_gated_act(void*, const void*, const void*, int64_t, int, int, float, float, float, int,
                           hipStream_t);
 void seq_launch_rope_pairs_store(void*, const void*, const void*, const int64_t*, const float*, void*, void*,
@@ -257,14 +257,17 @@ void sandwich_residual(torch::Tensor x, torch::Tensor a, torch::Tensor b, torch:
                                want ? out.data_ptr() : nullptr, T, W, (float)eps, f32flag(a), cur_stream());
 }
 
-void gated_rmsnorm(torch::Tensor out, torch::Tensor o, torch::Tensor w, torch::Tensor gate, double eps) {
+// gate_first: out = rms(o * silu(gate)) * w with w [G * S]; else out = rms(o) * w * sigmoid(gate) with w [S]
+void gated_rmsnorm(torch::Tensor out, torch::Tensor o, torch::Tensor w, torch::Tensor gate, double eps,
+                   bool gate_first) {
   CHECK_ACT(out); CHECK_F32C(o); CHECK_F32C(w); CHECK_ACT(gate); CHECK_SAME(gate, out); CHECK_ROWS2(gate);
   TORCH_CHECK(o.dim() == 3 && out.is_contiguous() && out.numel() == o.numel());
   const int T = o.size(0), G = o.size(1), S = o.size(2);
-  TORCH_CHECK(w.numel() == S && gate.size(0) == T && gate.size(1) == (int64_t)G * S);
+  TORCH_CHECK(w.numel() == (gate_first ? (int64_t)G * S : S) && gate.size(0) == T &&
+              gate.size(1) == (int64_t)G * S);
   if (T == 0) return;
   seq_launch_gated_rmsnorm(out.data_ptr(), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(), T, G, S,
-                           (int)gate.stride(0), (float)eps, f32flag(out), cur_stream());
+                           (int)gate.stride(0), (float)eps, gate_first ? 1 : 0, f32flag(out), cur_stream());
 }
 
 void gated_act(torch::Tensor out, torch::Tensor gate, torch::Tensor up, double limit, double alpha,
@@ -579,8 +582,7 @@ void head_rmsnorm_gate(torch::Tensor out, torch::Tensor o, torch::Tensor w, torc
   const int T = o.size(0), H = o.size(1), S = (int)o.size(2) - (ext ? 1 : 0);
   TORCH_CHECK(S >= 1 && out.numel() == (int64_t)T * H * S);
   TORCH_CHECK(w.numel() == (int64_t)H * S && gate.size(0) == T && gate.size(1) == (int64_t)H * S);
-  TORCH_CHECK(gate_act >= 0 && gate_act <= 2, "gate_act: 0 = sigmoid, 1 = silu, 2 = silu before the norm");
-  TORCH_CHECK(gate_act != 2 || !ext);
+  TORCH_CHECK(gate_act == 0 || gate_act == 1, "gate_act: 0 = sigmoid, 1 = silu");
   if (ext) { CHECK_F32C(mt); TORCH_CHECK(mt.numel() == (int64_t)T * H); }
   if (T == 0) return;
   seq_launch_head_rmsnorm_gate(out.data_ptr(), o.data_ptr<float>(), w.data_ptr<float>(), gate.data_ptr(),

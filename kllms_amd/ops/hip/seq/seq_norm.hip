@@ -159,21 +159,30 @@ __global__ void sandwich_residual_v8_kernel(float* __restrict__ x, const T* __re
 }
 
 // out[t, g*S + i] = o[t,g,i] / rms(o[t,g,:]) * w[i] * sigmoid(gate[t, g*S + i])
+// gate_first: the gate is silu and comes before the norm, the weight spans the
+// whole row: y = o * silu(gate); out = y / rms(y[t,g,:]) * w[g*S + i]
 template <typename T>
 __global__ void gated_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ o,
                                      const float* __restrict__ w, const T* __restrict__ gate,
-                                     int S, int gate_stride, float eps) {
+                                     int S, int gate_stride, float eps, int gate_first) {
   __shared__ float scratch[16];
   const int t = blockIdx.x, g = blockIdx.y, G = gridDim.y;
   const float* row = o + ((int64_t)t * G + g) * S;
+  const T* grow = gate + (int64_t)t * gate_stride + (int64_t)g * S;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < S; i += blockDim.x) { float v = row[i]; ss += v * v; }
+  for (int i = threadIdx.x; i < S; i += blockDim.x) {
+    float v = row[i];
+    if (gate_first) v *= silu_exact(ldf(grow + i));
+    ss += v * v;
+  }
   ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)S + eps);
-  const T* grow = gate + (int64_t)t * gate_stride + (int64_t)g * S;
   T* orow = out + ((int64_t)t * G + g) * S;
-  for (int i = threadIdx.x; i < S; i += blockDim.x)
-    stf(orow + i, row[i] * r * w[i] * sigmoid_exact(ldf(grow + i)));
+  for (int i = threadIdx.x; i < S; i += blockDim.x) {
+    const float gv = ldf(grow + i);
+    stf(orow + i, gate_first ? row[i] * silu_exact(gv) * r * w[(int64_t)g * S + i]
+                             : row[i] * r * w[i] * sigmoid_exact(gv));
+  }
 }
 
 // 8-wide, single pass: each thread keeps its (up to two) chunks of the row in
@@ -181,10 +190,11 @@ __global__ void gated_rmsnorm_kernel(T* __restrict__ out, const float* __restric
 template <typename T>
 __global__ void gated_rmsnorm_v8_kernel(T* __restrict__ out, const float* __restrict__ o,
                                         const float* __restrict__ w, const T* __restrict__ gate,
-                                        int S, int gate_stride, float eps) {
+                                        int S, int gate_stride, float eps, int gate_first) {
   __shared__ float scratch[16];
   const int t = blockIdx.x, g = blockIdx.y, G = gridDim.y;
   const float* row = o + ((int64_t)t * G + g) * S;
+  const T* grow = gate + (int64_t)t * gate_stride + (int64_t)g * S;
   float v[2][8], ww[8], gg[8];
   float ss = 0.f;
 #pragma unroll
@@ -192,21 +202,31 @@ __global__ void gated_rmsnorm_v8_kernel(T* __restrict__ out, const float* __rest
     const int i = (threadIdx.x + c * blockDim.x) * 8;
     if (i < S) {
       ld8(row + i, v[c]);
+      if (gate_first) {
+        ld8(grow + i, gg);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[c][e] *= silu_exact(gg[e]);
+      }
 #pragma unroll
       for (int e = 0; e < 8; ++e) ss += v[c][e] * v[c][e];
     }
   }
   ss = block_sum(ss, scratch);
   const float r = 1.0f / sqrtf(ss / (float)S + eps);
-  const T* grow = gate + (int64_t)t * gate_stride + (int64_t)g * S;
   T* orow = out + ((int64_t)t * G + g) * S;
 #pragma unroll
   for (int c = 0; c < 2; ++c) {
     const int i = (threadIdx.x + c * blockDim.x) * 8;
     if (i < S) {
-      ld8(w + i, ww); ld8(grow + i, gg);
+      if (gate_first) {
+        ld8(w + (int64_t)g * S + i, ww);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[c][e] = v[c][e] * r * ww[e] * sigmoid_exact(gg[e]);
+        for (int e = 0; e < 8; ++e) v[c][e] = v[c][e] * r * ww[e];
+      } else {
+        ld8(w + i, ww); ld8(grow + i, gg);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[c][e] = v[c][e] * r * ww[e] * sigmoid_exact(gg[e]);
+      }
       st8(orow + i, v[c]);
     }
   }
@@ -217,27 +237,32 @@ __global__ void gated_rmsnorm_v8_kernel(T* __restrict__ out, const float* __rest
 template <typename T>
 __global__ void gated_rmsnorm_rows_kernel(T* __restrict__ out, const float* __restrict__ o,
                                           const float* __restrict__ w, const T* __restrict__ gate,
-                                          int64_t rows, int G, int S, int LPG, int gate_stride, float eps) {
+                                          int64_t rows, int G, int S, int LPG, int gate_stride, float eps,
+                                          int gate_first) {
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t row = tid / LPG;
   const int i = (int)(tid - row * LPG) * 8;
   const bool on = row < rows;
+  const int64_t t = row / G;
+  const int g = (int)(row - t * G);
   float v[8], ww[8], gg[8];
   float ss = 0.f;
   if (on) {
     ld8(o + row * S + i, v);
+    ld8(gate + t * gate_stride + (int64_t)g * S + i, gg);
+    if (gate_first) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] *= silu_exact(gg[e]);
+    }
 #pragma unroll
     for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
   }
   for (int off = 1; off < LPG; off <<= 1) ss += __shfl_xor(ss, off);
   if (!on) return;
   const float r = 1.0f / sqrtf(ss / (float)S + eps);
-  const int64_t t = row / G;
-  const int g = (int)(row - t * G);
-  ld8(w + i, ww);
-  ld8(gate + t * gate_stride + (int64_t)g * S + i, gg);
+  ld8(w + (gate_first ? (int64_t)g * S : 0) + i, ww);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) v[e] = v[e] * r * ww[e] * sigmoid_exact(gg[e]);
+  for (int e = 0; e < 8; ++e) v[e] = v[e] * r * ww[e] * (gate_first ? 1.0f : sigmoid_exact(gg[e]));
   st8(out + row * S + i, v);
 }
 
@@ -371,28 +396,28 @@ extern "C" void seq_launch_sandwich_residual(float* x, const void* a, const void
 }
 
 extern "C" void seq_launch_gated_rmsnorm(void* out, const float* o, const float* w, const void* gate,
-                                         int T_, int G, int S, int gate_stride, float eps, int is_f32,
-                                         hipStream_t st) {
+                                         int T_, int G, int S, int gate_stride, float eps, int gate_first,
+                                         int is_f32, hipStream_t st) {
   if (S % 8 == 0 && gate_stride % 8 == 0 && aligned16(out) && aligned16(o) && aligned16(w) && aligned16(gate)) {
     const int lpg = S / 8;
     if (lpg <= 64 && (lpg & (lpg - 1)) == 0) {
       const int64_t rows = (int64_t)T_ * G;
       const int grid = (int)((rows * lpg + 255) / 256);
       DISPATCH_T(is_f32, hipLaunchKernelGGL(gated_rmsnorm_rows_kernel<T>, dim3(grid), dim3(256), 0, st, (T*)out,
-                                            o, w, (const T*)gate, rows, G, S, lpg, gate_stride, eps);)
+                                            o, w, (const T*)gate, rows, G, S, lpg, gate_stride, eps, gate_first);)
       return;
     }
     int threads = ((lpg + 1) / 2 + WAVE - 1) / WAVE * WAVE;       // two chunks of 8 per thread
     if (threads <= 1024) {
       if (threads < WAVE) threads = WAVE;
       DISPATCH_T(is_f32, hipLaunchKernelGGL(gated_rmsnorm_v8_kernel<T>, dim3(T_, G), dim3(threads), 0, st,
-                                            (T*)out, o, w, (const T*)gate, S, gate_stride, eps);)
+                                            (T*)out, o, w, (const T*)gate, S, gate_stride, eps, gate_first);)
       return;
     }
   }
   const int threads = S >= 256 ? 256 : (S > 64 ? 128 : 64);
   DISPATCH_T(is_f32, hipLaunchKernelGGL(gated_rmsnorm_kernel<T>, dim3(T_, G), dim3(threads), 0, st, (T*)out,
-                                        o, w, (const T*)gate, S, gate_stride, eps);)
+                                        o, w, (const T*)gate, S, gate_stride, eps, gate_first);)
 }
 
 extern "C" void seq_launch_gated_act(void* out, const void* gate, const void* up, int64_t rows, int cols,

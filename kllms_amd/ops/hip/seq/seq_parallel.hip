@@ -165,8 +165,7 @@ __global__ void cast_concat_kernel(T* __restrict__ out, float* __restrict__ x, c
 
 // ---- per-head RMS norm, full-width weight, activated gate ------------------------
 // o [T, H, S] fp32; out[t, h*S + i] = o / rms(o[t,h,:]) * w[h*S + i] * act(gate[t, h*S + i]);
-// act = sigmoid (0) or silu (1); 2: the silu gate is applied BEFORE the norm,
-// out = rms(o * silu(gate)) * w. One wave per (row, head). With mt != nullptr the
+// act = sigmoid (0) or silu (1). One wave per (row, head). With mt != nullptr the
 // head rows of o are S + 1 wide: the last entry is a normaliser n.q and the
 // head is first divided by max(|n.q|, e^-mt) + 1e-6 (the mlstm read-out).
 template <typename T>
@@ -178,21 +177,11 @@ __global__ void head_rmsnorm_gate_kernel(T* __restrict__ out, const float* __res
   const int h = blockIdx.y, lane = threadIdx.x;
   const float* orow = o + (t * H + h) * (mt != nullptr ? S + 1 : S);
   const float pre = mt != nullptr ? 1.0f / (fmaxf(fabsf(orow[S]), expf(-mt[t * H + h])) + 1e-6f) : 1.0f;
-  const T* grow = gate + t * gate_stride + (int64_t)h * S;
-  if (gate_act == 2) {
-    // the gate comes first: rms(o * silu(g)) * w
-    float ss = 0.f;
-    for (int i = lane; i < S; i += WAVE) { const float v = orow[i] * silu_exact(ldf(grow + i)); ss += v * v; }
-    ss = wave_sum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)S + eps);
-    for (int i = lane; i < S; i += WAVE)
-      stf(out + (t * H + h) * S + i, orow[i] * silu_exact(ldf(grow + i)) * r * w[(int64_t)h * S + i]);
-    return;
-  }
   float ss = 0.f;
   for (int i = lane; i < S; i += WAVE) { const float v = orow[i] * pre; ss += v * v; }
   ss = wave_sum(ss);
   const float r = pre / sqrtf(ss / (float)S + eps);
+  const T* grow = gate + t * gate_stride + (int64_t)h * S;
   for (int i = lane; i < S; i += WAVE) {
     const float g = ldf(grow + i);
     const float ga = gate_act == 0 ? sigmoid_exact(g) : silu_exact(g);
