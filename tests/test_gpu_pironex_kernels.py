@@ -186,6 +186,29 @@ def test_pooled_runs_update_and_attention(dtype, G, D, Dv, BS, run):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,Dv", [(8, 2, 128, 128), (16, 2, 64, 32), (4, 2, 32, 64), (8, 8, 16, 16), (6, 2, 64, 64),
+                                      (8, 1, 32, 256)])
+def test_window_attention_with_grouped_queries(dtype, H, G, D, Dv):
+    """1, 2, 3, 4 and 8 query heads per key/value head, key and value sizes
+    from 16 to 256, with and without key shares."""
+    BS, run, size, ctx, n_seq = 16, 5, 70, 300, 2
+    bt, kc, vc = paged(ctx, G, D, Dv, BS, dtype, n_seq, seed=H)
+    NB, PB = kc.shape[0], (BS + run - 1) // run
+    pk, pv = torch.zeros(NB, G, PB, D, device=DEV), torch.zeros(NB, G, PB, Dv, device=DEV)
+    pos = torch.arange(ctx, device=DEV).repeat(n_seq)
+    tseg = torch.arange(n_seq, device=DEV).repeat_interleave(ctx).int()
+    torch_ref.pool_kv_update(kc, vc, pk, pv, bt, tseg, pos, run)
+    rows = [(0, 0), (1, 3), (0, 69), (0, 70), (1, 74), (1, 75), (0, 299), (1, 200), (1, 201), (1, 202), (0, 150)]
+    ts = i32([s_ for s_, _ in rows])
+    ps = torch.tensor([p_ for _, p_ in rows], device=DEV)
+    q = rnd(len(rows), H, D, dtype=dtype, seed=3, std=1.2)
+    want = torch_ref.attn_window_pool_paged(q, kc, vc, pk, pv, bt, ts, ps, 0.25, 8.0, size, run)
+    for splits in (1, 0, 3):
+        close(ops.attn_window_pool_paged(q, kc, vc, pk, pv, bt, ts, ps, 0.25, 8.0, size, run, key_splits=splits),
+              want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C,K,stride", [(40, 4, 48), (37, 3, 37), (480, 4, 488), (16, 1, 16)])
 def test_causal_conv_with_bias(dtype, C, K, stride):
     lengths, starts, slots = [6, 1, 2, 1], [0, 5, 9, 0], [1, 3, 0, 2]
